@@ -1,0 +1,396 @@
+// Bag reduction (sum / mean / max / square-sum, optional per-sample weights), fixed-length
+// bags and plain row gather for gfx950.
+//
+// Work decomposition
+//   * A table row is read with 128-bit loads: a row of `dim` elements needs dim*sizeof(T)/16
+//     lanes.  G = that number rounded up to a power of two (at most 64) lanes form a
+//     sub-wavefront "slot"; a 256-lane workgroup holds 256/G slots, each reducing one bag at
+//     a time with fp32 accumulators in registers.  Rows wider than 1 KiB are cut into column
+//     slices of 64 lanes and a (bag, slice) pair becomes the unit of work.
+//   * A workgroup owns a contiguous run of bags.  Their offsets, and the ids (and weights)
+//     they cover, are copied into LDS once with coalesced loads; slots then read ids from
+//     LDS as broadcasts, so the only per-row global traffic is the row itself.
+//   * Slots pull the next bag of the run from an LDS counter, which evens out the long tail
+//     of bag lengths inside a workgroup.
+//   * Rows of one bag are added strictly in bag order (eight loads in flight, consumed in
+//     order), so fp32 results do not depend on the launch shape.
+//
+// Memory safety: offsets are clamped to [0, input_size] and made non-decreasing before use,
+// ids outside [data_offset, data_offset+count) never form an address, so arbitrary input
+// bytes cannot make the kernel read or write out of bounds.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "../common.h"
+
+namespace fwdmi {
+namespace {
+
+constexpr int kWG = 256;           // lanes per workgroup
+constexpr int kIdxCap = 2048;      // ids staged in LDS per workgroup
+constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
+constexpr int kUnroll = 8;         // row loads in flight per lane
+
+enum Kind { kPlain = 0, kWeighted = 1, kMax = 2 };
+
+struct BagLaunch {
+  const fwdmi_bag_table* tables;  // device array, or nullptr -> `single`
+  fwdmi_bag_table single;
+  const void* psw;  // per-sample weights (single-table form only)
+  void* out;
+  void* max_indices;
+  int32_t* oob_flag;
+  int64_t n_bags;
+  int64_t out_stride;
+  int64_t fixed_len;  // >= 0: bag b covers ids [b*fixed_len, (b+1)*fixed_len); < 0: use offsets
+  int32_t dim;
+  int32_t op;
+  int32_t out_f16;
+  int32_t include_last;
+  int32_t log2_g;
+  int32_t n_slices;
+  int32_t bags_per_wg;
+  int32_t wgs_per_table;
+  int32_t vec_store;
+};
+
+template <typename T, int N>
+struct alignas((sizeof(T) * N) < 16 ? (sizeof(T) * N) : 16) Pack {
+  T v[N];
+};
+
+template <typename TW, typename TI, int VEC, int KIND>
+__global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
+  __shared__ int64_t s_off[kMaxBagsPerWG + 1];
+  __shared__ TI s_idx[kIdxCap];
+  __shared__ float s_w[KIND == kWeighted ? kIdxCap : 1];
+  __shared__ int s_next;
+
+  const int tid = threadIdx.x;
+  const int t = blockIdx.x / L.wgs_per_table;
+  const int wg = blockIdx.x - t * L.wgs_per_table;
+  const fwdmi_bag_table T = L.tables ? L.tables[t] : L.single;
+
+  const int G = 1 << L.log2_g;
+  const int slot = tid >> L.log2_g;
+  const int gl = tid & (G - 1);
+  const int slots = kWG >> L.log2_g;
+
+  const int64_t bag0 = (int64_t)wg * L.bags_per_wg;
+  const int nb = (int)min((int64_t)L.bags_per_wg, L.n_bags - bag0);
+  const TI* __restrict__ ids = static_cast<const TI*>(T.input);
+  const TW* __restrict__ psw = static_cast<const TW*>(L.psw);
+
+  // ---- stage the run's offsets (clamped) ------------------------------------------------
+  for (int i = tid; i <= nb; i += kWG) {
+    int64_t v;
+    if (L.fixed_len >= 0) {
+      v = (bag0 + i) * L.fixed_len;
+    } else {
+      const int64_t b = bag0 + i;
+      v = (b < L.n_bags || L.include_last) ? (int64_t) static_cast<const TI*>(T.input_2)[b]
+                                           : T.input_size;
+    }
+    s_off[i] = min(max(v, (int64_t)0), T.input_size);
+  }
+  if (tid == 0) s_next = slots;
+  __syncthreads();
+
+  // ---- stage the ids (and weights) the run covers ----------------------------------------
+  const int64_t span0 = s_off[0];
+  const int64_t span = s_off[nb] - span0;
+  const bool staged = span >= 0 && span <= kIdxCap;  // uniform over the workgroup
+  if (staged) {
+    for (int i = tid; i < span; i += kWG) {
+      s_idx[i] = ids[span0 + i];
+      if (KIND == kWeighted) s_w[i] = (float)psw[span0 + i];
+    }
+  }
+  __syncthreads();
+
+  const TW* __restrict__ tab = static_cast<const TW*>(T.data);
+  const int n_units = nb * L.n_slices;
+  const bool square = L.op == FWDMI_OP_SQUARE_SUM;
+  bool oob = false;
+
+  int unit = slot;
+  while (unit < n_units) {
+    const int lb = L.n_slices == 1 ? unit : unit / L.n_slices;
+    const int sl = unit - lb * L.n_slices;
+    const int64_t start = s_off[lb];
+    const int64_t end = max(s_off[lb + 1], start);
+    const int col = (sl * G + gl) * VEC;
+    const bool col_ok = col < L.dim;
+    const int col_c = col_ok ? col : 0;
+    // A run whose offsets decrease can make [start,end) leave the staged window.
+    const bool in_lds = staged && start >= span0 && end <= span0 + span;
+
+    float acc[VEC];
+    TI arg[KIND == kMax ? VEC : 1];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < (KIND == kMax ? VEC : 1); ++e) arg[e] = 0;
+    bool first = true;
+
+    // Loads `UU` rows starting at bag position i, then folds them in order.
+    auto step = [&](auto uu_tag, int64_t i) {
+      constexpr int UU = decltype(uu_tag)::value;
+      Pack<TW, VEC> v[UU];
+      TI id[UU];
+      float w[UU];
+      bool ok[UU];
+#pragma unroll
+      for (int u = 0; u < UU; ++u) {
+        const int64_t p = i + u;
+        id[u] = in_lds ? s_idx[p - span0] : ids[p];
+        if (KIND == kWeighted) w[u] = in_lds ? s_w[p - span0] : (float)psw[p];
+        const uint64_t row = (uint64_t)((int64_t)id[u] - T.data_offset);
+        ok[u] = row < (uint64_t)T.count;
+        oob |= !ok[u];
+        const uint64_t row_c = ok[u] ? row : 0;  // never form an address from a bad id
+        v[u] = *reinterpret_cast<const Pack<TW, VEC>*>(tab + row_c * (uint64_t)L.dim + col_c);
+      }
+#pragma unroll
+      for (int u = 0; u < UU; ++u) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float x = ok[u] ? (float)v[u].v[e] : 0.0f;
+          if (KIND == kPlain) {
+            acc[e] = square ? __builtin_fmaf(x, x, acc[e]) : acc[e] + x;
+          } else if (KIND == kWeighted) {
+            acc[e] = __builtin_fmaf(ok[u] ? w[u] : 0.0f, x, acc[e]);
+          } else {
+            if (ok[u] && (first || x > acc[e])) {
+              acc[e] = x;
+              arg[e] = id[u];
+            }
+          }
+        }
+        if (KIND == kMax && ok[u]) first = false;
+      }
+    };
+
+    int64_t i = start;
+    for (; i + kUnroll <= end; i += kUnroll) step(std::integral_constant<int, kUnroll>{}, i);
+    if (i + 4 <= end) {
+      step(std::integral_constant<int, 4>{}, i);
+      i += 4;
+    }
+    if (i + 2 <= end) {
+      step(std::integral_constant<int, 2>{}, i);
+      i += 2;
+    }
+    if (i < end) step(std::integral_constant<int, 1>{}, i);
+
+    // ---- epilogue: mean scaling, store ---------------------------------------------------
+    const int64_t len = end - start;
+    if (L.op == FWDMI_OP_MEAN && len > 0) {
+      const float flen = (float)len;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] = acc[e] / flen;
+    }
+    if (col_ok) {
+      const int64_t o = (bag0 + lb) * L.out_stride + T.out_col + col;
+      if (L.out_f16) {
+        _Float16* op = static_cast<_Float16*>(L.out) + o;
+        if (L.vec_store) {
+          Pack<_Float16, VEC> r;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) r.v[e] = (_Float16)acc[e];
+          *reinterpret_cast<Pack<_Float16, VEC>*>(op) = r;
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) op[e] = (_Float16)acc[e];
+        }
+      } else {
+        float* op = static_cast<float*>(L.out) + o;
+        if (L.vec_store) {
+          Pack<float, VEC> r;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) r.v[e] = acc[e];
+          *reinterpret_cast<Pack<float, VEC>*>(op) = r;
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) op[e] = acc[e];
+        }
+      }
+      if (KIND == kMax && L.max_indices) {
+        TI* mp = static_cast<TI*>(L.max_indices) + (bag0 + lb) * (int64_t)L.dim + col;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) mp[e] = arg[e];
+      }
+    }
+
+    // ---- next unit of the run ------------------------------------------------------------
+    int nxt = 0;
+    if (gl == 0) nxt = atomicAdd(&s_next, 1);
+    unit = __shfl(nxt, 0, G);
+  }
+
+  if (oob && L.oob_flag) atomicOr(L.oob_flag, 1);
+}
+
+template <typename TW, typename TI, int VEC>
+int launch_kind(int kind, const BagLaunch& L, int grid, hipStream_t stream) {
+  switch (kind) {
+    case kPlain:
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kPlain>), dim3(grid), dim3(kWG), 0, stream, L);
+      break;
+    case kWeighted:
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kWeighted>), dim3(grid), dim3(kWG), 0, stream, L);
+      break;
+    default:
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMax>), dim3(grid), dim3(kWG), 0, stream, L);
+  }
+  FWDMI_HIP_CHECK(hipGetLastError());
+  return FWDMI_OK;
+}
+
+template <typename TW, typename TI>
+int launch_vec(bool vec, int kind, const BagLaunch& L, int grid, hipStream_t stream) {
+  constexpr int kVec = 16 / sizeof(TW);
+  return vec ? launch_kind<TW, TI, kVec>(kind, L, grid, stream)
+             : launch_kind<TW, TI, 1>(kind, L, grid, stream);
+}
+
+int next_pow2(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+// Validates arguments, picks the lane mapping and launches.  `tables_dev` non-null selects the
+// multi-table form (then `single` is only used for host-side checks of shared fields).
+int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_bag_table& single,
+                 void* output, int64_t n_bags, int64_t fixed_len, int dim, int op, double avg_len,
+                 const fwdmi_bag_ext* ext, hipStream_t stream) {
+  clear_error();
+  static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr};
+  const fwdmi_bag_ext& x = ext ? *ext : kDefaultExt;
+
+  if (!is_float_dtype(x.table_dtype) || !is_float_dtype(x.out_dtype) || !is_index_dtype(x.index_dtype))
+    return set_error(FWDMI_ERR_UNSUPPORTED, "embedding bag: unsupported dtype (table %d, index %d, out %d)",
+                     x.table_dtype, x.index_dtype, x.out_dtype);
+  if (op != FWDMI_OP_SUM && op != FWDMI_OP_MEAN && op != FWDMI_OP_MAX && op != FWDMI_OP_SQUARE_SUM)
+    return set_error(FWDMI_ERR_UNSUPPORTED, "embedding bag: unknown op %d", op);
+  FWDMI_REQUIRE(n_bags >= 0 && dim > 0 && n_tables > 0, "embedding bag: n_bags=%lld dim=%d n_tables=%d",
+                (long long)n_bags, dim, n_tables);
+  FWDMI_REQUIRE(!x.per_sample_weights || op == FWDMI_OP_SUM,
+                "embedding bag: per_sample_weights needs op SUM (got %d)", op);
+  FWDMI_REQUIRE(!x.max_indices || (op == FWDMI_OP_MAX && !tables_dev),
+                "embedding bag: max_indices needs op MAX on a single table");
+  const int64_t out_stride = x.out_row_stride > 0 ? x.out_row_stride : dim;
+  FWDMI_REQUIRE(out_stride >= dim, "embedding bag: out_row_stride %lld < dim %d", (long long)out_stride, dim);
+  if (n_bags == 0) return FWDMI_OK;
+  FWDMI_REQUIRE(output != nullptr, "embedding bag: null output");
+  if (!tables_dev) {
+    FWDMI_REQUIRE(single.count > 0 && single.data, "embedding bag: empty table");
+    FWDMI_REQUIRE(single.input_size >= 0 && (single.input_size == 0 || single.input),
+                  "embedding bag: null ids");
+    FWDMI_REQUIRE(fixed_len >= 0 || single.input_2, "embedding bag: null offsets");
+    FWDMI_REQUIRE(single.out_col >= 0 && single.out_col + dim <= out_stride, "embedding bag: out_col");
+  }
+
+  const size_t sw = dtype_size(x.table_dtype), so = dtype_size(x.out_dtype);
+  const int vec_w = (int)(16 / sw);
+  // 128-bit row loads need 16-byte row pitch and base; a multi-table launch is checked by its caller.
+  bool vec = (dim % vec_w) == 0;
+  if (!tables_dev) vec = vec && (reinterpret_cast<uintptr_t>(single.data) % 16) == 0;
+  const int VEC = vec ? vec_w : 1;
+
+  BagLaunch L{};
+  L.tables = tables_dev;
+  L.single = single;
+  L.out = output;
+  L.max_indices = x.max_indices;
+  L.oob_flag = x.oob_flag;
+  L.n_bags = n_bags;
+  L.out_stride = out_stride;
+  L.fixed_len = fixed_len;
+  L.dim = dim;
+  L.op = op;
+  L.out_f16 = x.out_dtype == FWDMI_F16;
+  L.include_last = x.include_last_offset != 0;
+  const int lanes = std::min(64, next_pow2((dim + VEC - 1) / VEC));
+  L.log2_g = __builtin_ctz(lanes);
+  L.n_slices = (dim + lanes * VEC - 1) / (lanes * VEC);
+  const int slots = kWG / lanes;
+  if (avg_len < 1.0) avg_len = 1.0;
+  int k = (int)(kIdxCap / 1.5 / (avg_len * slots));
+  k = std::max(1, std::min(8, k));
+  L.bags_per_wg = std::max(1, std::min(kMaxBagsPerWG, slots * k / L.n_slices));
+  const int64_t wgs = (n_bags + L.bags_per_wg - 1) / L.bags_per_wg;
+  FWDMI_REQUIRE(wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
+  L.wgs_per_table = (int)wgs;
+  const size_t store_align = std::min<size_t>(16, VEC * so);
+  L.vec_store = VEC > 1 && (reinterpret_cast<uintptr_t>(output) % store_align) == 0 &&
+                ((out_stride * so) % store_align) == 0 &&
+                (tables_dev || (single.out_col * so) % store_align == 0);
+
+  const int kind = op == FWDMI_OP_MAX ? kMax : (x.per_sample_weights ? kWeighted : kPlain);
+  L.psw = x.per_sample_weights;
+  const int grid = (int)(wgs * n_tables);
+  const bool f16 = x.table_dtype == FWDMI_F16, i64 = x.index_dtype == FWDMI_I64;
+  if (f16)
+    return i64 ? launch_vec<_Float16, int64_t>(vec, kind, L, grid, stream)
+               : launch_vec<_Float16, int32_t>(vec, kind, L, grid, stream);
+  return i64 ? launch_vec<float, int64_t>(vec, kind, L, grid, stream)
+             : launch_vec<float, int32_t>(vec, kind, L, grid, stream);
+}
+
+}  // namespace
+}  // namespace fwdmi
+
+extern "C" {
+
+int fwdmi_embedding_bag(const void* input, const void* input_2, void* output, int64_t input_size,
+                        int64_t block_size, const void* data, int64_t count, int32_t dim,
+                        int64_t data_offset, int32_t op_type, const fwdmi_bag_ext* ext, void* stream) {
+  fwdmi_bag_table t{data, input, input_2, count, input_size, data_offset, 0};
+  const double avg = block_size > 0 ? (double)input_size / (double)block_size : 1.0;
+  return fwdmi::bag_dispatch(nullptr, 1, t, output, block_size, -1, dim, op_type, avg, ext,
+                             static_cast<hipStream_t>(stream));
+}
+
+int fwdmi_embedding_bag_fixed(const void* input, void* output, int64_t batch_size, int64_t offset,
+                              const void* data, int64_t count, int32_t dim, int64_t data_offset,
+                              int32_t op_type, const fwdmi_bag_ext* ext, void* stream) {
+  if (offset < 0 || batch_size < 0)
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "fixed-length bags: batch %lld x length %lld",
+                            (long long)batch_size, (long long)offset);
+  fwdmi_bag_table t{data, input, nullptr, count, batch_size * offset, data_offset, 0};
+  return fwdmi::bag_dispatch(nullptr, 1, t, output, batch_size, offset, dim, op_type, (double)offset, ext,
+                             static_cast<hipStream_t>(stream));
+}
+
+int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t offset, const void* data,
+                 int64_t count, int32_t dim, int64_t data_offset, const fwdmi_bag_ext* ext, void* stream) {
+  if (offset < 0 || batch_size < 0)
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "gather: batch %lld x %lld", (long long)batch_size,
+                            (long long)offset);
+  // A gather is a sum over bags of exactly one id.
+  fwdmi_bag_ext x = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr};
+  x.per_sample_weights = nullptr;
+  x.max_indices = nullptr;
+  x.out_row_stride = 0;
+  const int64_t n = batch_size * offset;
+  fwdmi_bag_table t{data, input, nullptr, count, n, data_offset, 0};
+  return fwdmi::bag_dispatch(nullptr, 1, t, output, n, 1, dim, FWDMI_OP_SUM, 1.0, &x,
+                             static_cast<hipStream_t>(stream));
+}
+
+int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_tables, int64_t n_bags,
+                              void* output, int32_t dim, int32_t op_type, double avg_bag_len,
+                              const fwdmi_bag_ext* ext, void* stream) {
+  if (!tables_dev) return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "multi-table bags: null table array");
+  if (ext && ext->per_sample_weights)
+    return fwdmi::set_error(FWDMI_ERR_UNSUPPORTED, "multi-table bags: per-sample weights are not supported");
+  fwdmi_bag_table none{};
+  return fwdmi::bag_dispatch(tables_dev, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, ext,
+                             static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,407 @@
+// LayerNorm family for gfx950: plain LayerNorm with optional pre-bias, SkipLayerNorm
+// (input + skip (+ bias)) and the BERT embedding lookup fused with LayerNorm (+ mask index).
+//
+// One wavefront owns one row.  Each lane keeps its 128-bit slices of the row in registers
+// (row read once), computes its own mean and centred sum of squares, and the 64 partial
+// (count, mean, M2) triples are merged with a butterfly of DPP row operations and two
+// cross-row shuffles (Chan's parallel Welford update), all in fp32.  gamma / beta (/ bias)
+// live in registers and are reused for every row the wavefront processes.
+//
+// Rows whose length or alignment rule out 128-bit access take the strided kernel: same
+// reduction, one element per lane per step, row read twice (the second time from cache).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+#include "../common.h"
+
+namespace fwdmi {
+namespace {
+
+constexpr int kWG = 256;
+constexpr int kWavesPerWG = kWG / 64;
+
+enum Mode { kLayerNorm = 0, kSkip = 1, kEmb = 2 };
+
+struct LnLaunch {
+  const void* input;  // kLayerNorm / kSkip: [rows, ld]; kEmb: word table
+  const void* skip;   // kSkip: [rows, ld]
+  const void* pos;    // kEmb
+  const void* tok;    // kEmb
+  const float* gamma;
+  const float* beta;
+  const float* bias;  // nullable
+  void* output;
+  const int32_t* input_ids;
+  const int32_t* segment_ids;
+  const int32_t* input_mask;
+  int32_t* mask_idx;
+  int32_t* oob_flag;
+  int64_t rows;
+  int32_t ld;
+  int32_t S, B;
+  int32_t word_count, pos_count, tok_count;
+  int32_t row_blocks;  // workgroups that process rows; the rest compute mask indices
+  int32_t total_waves; // row-processing wavefronts in the grid
+  float eps;
+};
+
+template <typename T, int N>
+struct alignas((sizeof(T) * N) < 16 ? (sizeof(T) * N) : 16) Pack {
+  T v[N];
+};
+
+struct Welford {
+  float n, mean, m2;
+};
+
+__device__ __forceinline__ Welford merge(const Welford a, const Welford b) {
+  Welford r;
+  r.n = a.n + b.n;
+  const float inv = r.n > 0.0f ? 1.0f / r.n : 0.0f;
+  const float d = b.mean - a.mean;
+  r.mean = a.mean + d * (b.n * inv);
+  r.m2 = a.m2 + b.m2 + d * d * (a.n * b.n * inv);
+  return r;
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+
+template <int CTRL>
+__device__ __forceinline__ Welford dpp(const Welford w) {
+  return Welford{dpp<CTRL>(w.n), dpp<CTRL>(w.mean), dpp<CTRL>(w.m2)};
+}
+
+__device__ __forceinline__ Welford xor_lanes(const Welford w, int mask) {
+  return Welford{__shfl_xor(w.n, mask), __shfl_xor(w.mean, mask), __shfl_xor(w.m2, mask)};
+}
+
+// After this every lane holds the statistics of all 64 lanes.
+__device__ __forceinline__ Welford wave_allreduce(Welford w) {
+  w = merge(w, dpp<0xB1>(w));   // quad_perm [1,0,3,2]: lane ^ 1
+  w = merge(w, dpp<0x4E>(w));   // quad_perm [2,3,0,1]: lane ^ 2
+  w = merge(w, dpp<0x141>(w));  // row_half_mirror: the other quad of each 8
+  w = merge(w, dpp<0x140>(w));  // row_mirror: the other half of each row of 16
+  w = merge(w, xor_lanes(w, 16));
+  w = merge(w, xor_lanes(w, 32));
+  // Lanes agree up to rounding (merge is not bitwise symmetric); take lane 0's value everywhere.
+  w.n = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(w.n)));
+  w.mean = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(w.mean)));
+  w.m2 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(w.m2)));
+  return w;
+}
+
+__device__ __forceinline__ int wave_min(int v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = min(v, __shfl_xor(v, m));
+  return v;
+}
+
+// Index of the first zero of mask column b ([S,B] layout), S when there is none.
+__device__ __forceinline__ void mask_index_wave(const LnLaunch& L, int b, int lane) {
+  int first = L.S;
+  for (int s = lane; s < L.S; s += 64)
+    if (L.input_mask[(int64_t)s * L.B + b] == 0) {
+      first = s;
+      break;
+    }
+  first = wave_min(first);
+  if (lane == 0) L.mask_idx[b] = first;
+}
+
+template <typename T, int VEC, int NV, int MODE>
+__global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
+  const int lane = threadIdx.x & 63;
+  const int wave_in_wg = threadIdx.x >> 6;
+  if ((int)blockIdx.x >= L.row_blocks) {
+    if (MODE == kEmb) {
+      const int b = ((int)blockIdx.x - L.row_blocks) * kWavesPerWG + wave_in_wg;
+      if (b < L.B) mask_index_wave(L, b, lane);
+    }
+    return;
+  }
+  const int wave = blockIdx.x * kWavesPerWG + wave_in_wg;
+
+  // Per-lane column slices: chunk j covers elements (j*64 + lane)*VEC .. +VEC.
+  bool live[NV];
+  float g[NV][VEC], be[NV][VEC], bi[NV][VEC];
+  float cnt = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = (j * 64 + lane) * VEC;
+    live[j] = c < L.ld;
+    const int cc = live[j] ? c : 0;
+    const Pack<float, VEC> pg = *reinterpret_cast<const Pack<float, VEC>*>(L.gamma + cc);
+    const Pack<float, VEC> pb = *reinterpret_cast<const Pack<float, VEC>*>(L.beta + cc);
+    Pack<float, VEC> pi{};
+    if (L.bias) pi = *reinterpret_cast<const Pack<float, VEC>*>(L.bias + cc);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      g[j][e] = pg.v[e];
+      be[j][e] = pb.v[e];
+      bi[j][e] = L.bias ? pi.v[e] : 0.0f;
+    }
+    if (live[j]) cnt += (float)VEC;
+  }
+  const float inv_cnt = cnt > 0.0f ? 1.0f / cnt : 0.0f;
+
+  bool oob = false;
+  for (int64_t r = wave; r < L.rows; r += L.total_waves) {
+    float x[NV][VEC];
+    if (MODE == kEmb) {
+      const int s = (int)(r / L.B);
+      const int64_t w = L.input_ids[r], sg = L.segment_ids[r];
+      const bool wok = w >= 0 && w < L.word_count, gok = sg >= 0 && sg < L.tok_count,
+                 pok = s < L.pos_count;
+      oob |= !(wok && gok && pok);
+      const T* wp = static_cast<const T*>(L.input) + (wok ? w : 0) * L.ld;
+      const T* pp = static_cast<const T*>(L.pos) + (int64_t)(pok ? s : 0) * L.ld;
+      const T* tp = static_cast<const T*>(L.tok) + (gok ? sg : 0) * L.ld;
+      Pack<T, VEC> a[NV], p[NV], q[NV];
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int cc = live[j] ? (j * 64 + lane) * VEC : 0;
+        a[j] = *reinterpret_cast<const Pack<T, VEC>*>(wp + cc);
+        p[j] = *reinterpret_cast<const Pack<T, VEC>*>(pp + cc);
+        q[j] = *reinterpret_cast<const Pack<T, VEC>*>(tp + cc);
+      }
+#pragma unroll
+      for (int j = 0; j < NV; ++j)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          x[j][e] = (wok ? (float)a[j].v[e] : 0.0f) + (pok ? (float)p[j].v[e] : 0.0f) +
+                    (gok ? (float)q[j].v[e] : 0.0f);
+    } else {
+      const T* ip = static_cast<const T*>(L.input) + r * L.ld;
+      const T* sp = static_cast<const T*>(L.skip) + r * L.ld;
+      Pack<T, VEC> a[NV], k[NV];
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int cc = live[j] ? (j * 64 + lane) * VEC : 0;
+        a[j] = *reinterpret_cast<const Pack<T, VEC>*>(ip + cc);
+        if (MODE == kSkip) k[j] = *reinterpret_cast<const Pack<T, VEC>*>(sp + cc);
+      }
+#pragma unroll
+      for (int j = 0; j < NV; ++j)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          float v = (float)a[j].v[e];
+          if (MODE == kSkip) v += (float)k[j].v[e];
+          x[j][e] = v + bi[j][e];
+        }
+    }
+
+    // lane-local statistics, then the wave-wide merge
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sum += live[j] ? x[j][e] : 0.0f;
+    Welford w{cnt, sum * inv_cnt, 0.0f};
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float d = live[j] ? x[j][e] - w.mean : 0.0f;
+        w.m2 = __builtin_fmaf(d, d, w.m2);
+      }
+    w = wave_allreduce(w);
+    const float mu = w.mean;
+    const float rs = 1.0f / sqrtf(w.m2 / w.n + L.eps);
+
+    T* op = static_cast<T*>(L.output) + r * L.ld;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      if (live[j]) {
+        Pack<T, VEC> o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o.v[e] = (T)(g[j][e] * ((x[j][e] - mu) * rs) + be[j][e]);
+        *reinterpret_cast<Pack<T, VEC>*>(op + (j * 64 + lane) * VEC) = o;
+      }
+    }
+  }
+  if (oob && L.oob_flag) atomicOr(L.oob_flag, 1);
+}
+
+// Any ld, any alignment: one element per lane per step, two passes over the row.
+template <typename T, int MODE>
+__global__ __launch_bounds__(kWG) void ln_strided_kernel(const LnLaunch L) {
+  const int lane = threadIdx.x & 63;
+  const int wave_in_wg = threadIdx.x >> 6;
+  if ((int)blockIdx.x >= L.row_blocks) {
+    if (MODE == kEmb) {
+      const int b = ((int)blockIdx.x - L.row_blocks) * kWavesPerWG + wave_in_wg;
+      if (b < L.B) mask_index_wave(L, b, lane);
+    }
+    return;
+  }
+  const int wave = blockIdx.x * kWavesPerWG + wave_in_wg;
+  bool oob = false;
+  for (int64_t r = wave; r < L.rows; r += L.total_waves) {
+    const T *p0 = nullptr, *p1 = nullptr, *p2 = nullptr;
+    bool ok0 = true, ok1 = false, ok2 = false;
+    if (MODE == kEmb) {
+      const int s = (int)(r / L.B);
+      const int64_t w = L.input_ids[r], sg = L.segment_ids[r];
+      ok0 = w >= 0 && w < L.word_count;
+      ok1 = s < L.pos_count;
+      ok2 = sg >= 0 && sg < L.tok_count;
+      oob |= !(ok0 && ok1 && ok2);
+      p0 = static_cast<const T*>(L.input) + (ok0 ? w : 0) * L.ld;
+      p1 = static_cast<const T*>(L.pos) + (int64_t)(ok1 ? s : 0) * L.ld;
+      p2 = static_cast<const T*>(L.tok) + (ok2 ? sg : 0) * L.ld;
+    } else {
+      p0 = static_cast<const T*>(L.input) + r * L.ld;
+      if (MODE == kSkip) {
+        p1 = static_cast<const T*>(L.skip) + r * L.ld;
+        ok1 = true;
+      }
+    }
+    auto fetch = [&](int i) {
+      float v = ok0 ? (float)p0[i] : 0.0f;
+      if (MODE != kLayerNorm) v += ok1 ? (float)p1[i] : 0.0f;
+      if (MODE == kEmb) v += ok2 ? (float)p2[i] : 0.0f;
+      if (MODE != kEmb && L.bias) v += L.bias[i];
+      return v;
+    };
+    Welford w{0.0f, 0.0f, 0.0f};
+    for (int i = lane; i < L.ld; i += 64) {
+      const float v = fetch(i);
+      w.n += 1.0f;
+      const float d = v - w.mean;
+      w.mean += d / w.n;
+      w.m2 = __builtin_fmaf(d, v - w.mean, w.m2);
+    }
+    w = wave_allreduce(w);
+    const float mu = w.mean;
+    const float rs = 1.0f / sqrtf(w.m2 / w.n + L.eps);
+    T* op = static_cast<T*>(L.output) + r * L.ld;
+    for (int i = lane; i < L.ld; i += 64) op[i] = (T)(L.gamma[i] * ((fetch(i) - mu) * rs) + L.beta[i]);
+  }
+  if (oob && L.oob_flag) atomicOr(L.oob_flag, 1);
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; }
+
+template <typename T, int MODE>
+int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
+  constexpr int kVec = 16 / sizeof(T);
+  static const int cus = [] {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      return v;
+    return 256;
+  }();
+  // Enough wavefronts to fill the chip; beyond that a wavefront loops over rows so the
+  // gamma/beta registers are reused.
+  const int64_t max_blocks = (int64_t)cus * 8;
+  const int64_t want = (L.rows + kWavesPerWG - 1) / kWavesPerWG;
+  L.row_blocks = (int)std::max<int64_t>(1, std::min(want, max_blocks));
+  L.total_waves = L.row_blocks * kWavesPerWG;
+  const int mask_blocks = (MODE == kEmb && L.mask_idx) ? (L.B + kWavesPerWG - 1) / kWavesPerWG : 0;
+  const dim3 grid(L.row_blocks + mask_blocks), block(kWG);
+
+  const int chunks = (L.ld + 64 * kVec - 1) / (64 * kVec);
+  if (vec_ok && (L.ld % kVec) == 0 && chunks <= 8) {
+    if (chunks <= 1)
+      hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 1, MODE>), grid, block, 0, stream, L);
+    else if (chunks <= 2)
+      hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 2, MODE>), grid, block, 0, stream, L);
+    else if (chunks <= 4)
+      hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 4, MODE>), grid, block, 0, stream, L);
+    else
+      hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 8, MODE>), grid, block, 0, stream, L);
+  } else {
+    hipLaunchKernelGGL((ln_strided_kernel<T, MODE>), grid, block, 0, stream, L);
+  }
+  FWDMI_HIP_CHECK(hipGetLastError());
+  return FWDMI_OK;
+}
+
+template <int MODE>
+int ln_dispatch(LnLaunch& L, int dtype, bool vec_ok, hipStream_t stream) {
+  if (dtype == FWDMI_F16) return ln_launch<_Float16, MODE>(L, vec_ok, stream);
+  if (dtype == FWDMI_F32) return ln_launch<float, MODE>(L, vec_ok, stream);
+  return set_error(FWDMI_ERR_UNSUPPORTED, "layer norm: unsupported dtype %d", dtype);
+}
+
+}  // namespace
+}  // namespace fwdmi
+
+extern "C" {
+
+int fwdmi_skip_layer_norm(void* stream, int32_t ld, int64_t n, const void* input, const void* skip,
+                          const float* beta, const float* gamma, void* output, const float* bias,
+                          int32_t dtype, float eps) {
+  using namespace fwdmi;
+  clear_error();
+  if (!is_float_dtype(dtype)) return set_error(FWDMI_ERR_UNSUPPORTED, "layer norm: unsupported dtype %d", dtype);
+  FWDMI_REQUIRE(ld > 0 && n >= 0 && n % ld == 0, "layer norm: n=%lld is not a multiple of ld=%d",
+                (long long)n, ld);
+  if (n == 0) return FWDMI_OK;
+  FWDMI_REQUIRE(input && output && beta && gamma, "layer norm: null pointer");
+  LnLaunch L{};
+  L.input = input;
+  L.skip = skip;
+  L.gamma = gamma;
+  L.beta = beta;
+  L.bias = bias;
+  L.output = output;
+  L.rows = n / ld;
+  L.ld = ld;
+  L.eps = eps;
+  const bool vec_ok = aligned16(input) && aligned16(output) && aligned16(gamma) && aligned16(beta) &&
+                      (!bias || aligned16(bias)) && (!skip || aligned16(skip));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return skip ? ln_dispatch<kSkip>(L, dtype, vec_ok, s) : ln_dispatch<kLayerNorm>(L, dtype, vec_ok, s);
+}
+
+int fwdmi_layer_norm(void* stream, int32_t ld, int64_t n, const void* input, const float* beta,
+                     const float* gamma, void* output, const float* bias, int32_t dtype, float eps) {
+  return fwdmi_skip_layer_norm(stream, ld, n, input, nullptr, beta, gamma, output, bias, dtype, eps);
+}
+
+int fwdmi_emb_layer_norm(void* stream, int32_t S, int32_t B, int32_t ld, const int32_t* input_ids,
+                         const int32_t* segment_ids, const int32_t* input_mask, const float* beta,
+                         const float* gamma, const void* word, const void* pos, const void* tok,
+                         int32_t word_count, int32_t pos_count, int32_t tok_count, void* output,
+                         int32_t* mask_idx, int32_t dtype, float eps, int32_t* oob_flag) {
+  using namespace fwdmi;
+  clear_error();
+  if (!is_float_dtype(dtype)) return set_error(FWDMI_ERR_UNSUPPORTED, "emb layer norm: unsupported dtype %d", dtype);
+  FWDMI_REQUIRE(S >= 0 && B >= 0 && ld > 0, "emb layer norm: S=%d B=%d ld=%d", S, B, ld);
+  if ((int64_t)S * B == 0) return FWDMI_OK;
+  FWDMI_REQUIRE(input_ids && segment_ids && beta && gamma && word && pos && tok && output,
+                "emb layer norm: null pointer");
+  FWDMI_REQUIRE(word_count > 0 && pos_count > 0 && tok_count > 0, "emb layer norm: empty table");
+  FWDMI_REQUIRE(!mask_idx || input_mask, "emb layer norm: mask_idx requested without input_mask");
+  LnLaunch L{};
+  L.input = word;
+  L.pos = pos;
+  L.tok = tok;
+  L.gamma = gamma;
+  L.beta = beta;
+  L.output = output;
+  L.input_ids = input_ids;
+  L.segment_ids = segment_ids;
+  L.input_mask = input_mask;
+  L.mask_idx = mask_idx;
+  L.oob_flag = oob_flag;
+  L.rows = (int64_t)S * B;
+  L.ld = ld;
+  L.S = S;
+  L.B = B;
+  L.word_count = word_count;
+  L.pos_count = pos_count;
+  L.tok_count = tok_count;
+  L.eps = eps;
+  const bool vec_ok = aligned16(word) && aligned16(pos) && aligned16(tok) && aligned16(output) &&
+                      aligned16(gamma) && aligned16(beta);
+  return ln_dispatch<kEmb>(L, dtype, vec_ok, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,206 @@
+"""Tensor-level wrappers of the kernel launchers in ``libfwdmi.so``.
+
+Each function validates that its operands are contiguous device tensors, allocates the output
+with torch (device memory plumbing only) and calls one C-ABI launcher on torch's current
+stream.  Nothing here computes: a missing GPU or library is an error, never a fallback.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import lib
+
+_FDT = {torch.float32: lib.F32, torch.float16: lib.F16}
+_IDT = {torch.int32: lib.I32, torch.int64: lib.I64}
+MODES = {"sum": lib.OP_SUM, "mean": lib.OP_MEAN, "max": lib.OP_MAX, "square_sum": lib.OP_SQUARE_SUM}
+
+
+def _dev(t, name):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise RuntimeError("%s must be a tensor in device memory (the HIP path has no CPU fallback)" % name)
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    return t
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _stream(stream):
+    s = torch.cuda.current_stream() if stream is None else stream
+    return C.c_void_p(s.cuda_stream)
+
+
+def _op(mode):
+    return MODES[mode] if isinstance(mode, str) else int(mode)
+
+
+def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_indices=None, out_row_stride=0,
+         oob_flag=None):
+    x = lib.BagExt()
+    x.table_dtype = _FDT[table.dtype]
+    x.index_dtype = _IDT[indices.dtype]
+    x.out_dtype = _FDT[out_dtype]
+    x.include_last_offset = 1 if include_last_offset else 0
+    x.per_sample_weights = psw.data_ptr() if psw is not None else None
+    x.max_indices = max_indices.data_ptr() if max_indices is not None else None
+    x.out_row_stride = int(out_row_stride)
+    x.oob_flag = oob_flag.data_ptr() if oob_flag is not None else None
+    return x
+
+
+def embedding_bag(table, indices, offsets, mode="sum", per_sample_weights=None, include_last_offset=False,
+                  data_offset=0, out_dtype=None, out=None, out_col=0, want_max_indices=False, oob_flag=None,
+                  count=None, stream=None):
+    """Bags over a 1-D ``indices`` + ``offsets`` layout -> ``[n_bags, dim]``.
+
+    ``out`` / ``out_col`` write a column block of an existing ``[n_bags, W]`` matrix.
+    Returns ``out`` or ``(out, max_indices)``.
+    """
+    table, indices, offsets = _dev(table, "table"), _dev(indices, "indices"), _dev(offsets, "offsets")
+    if indices.dtype != offsets.dtype:
+        raise TypeError("indices and offsets must share an integer dtype")
+    offsets = offsets.reshape(-1)
+    dim = table.shape[1]
+    n_bags = offsets.numel() - (1 if include_last_offset else 0)
+    odt = table.dtype if out_dtype is None else out_dtype
+    stride = 0
+    if out is None:
+        out = torch.empty((n_bags, dim), dtype=odt, device=table.device)
+        dst = out
+    else:
+        _dev(out, "out")
+        assert out.dtype == odt and out.shape[0] == n_bags
+        stride = out.shape[1]
+        dst = out.reshape(-1)[out_col:]
+    psw = None
+    if per_sample_weights is not None:
+        psw = _dev(per_sample_weights, "per_sample_weights")
+        assert psw.dtype == table.dtype and psw.numel() == indices.numel()
+    mi = torch.empty((n_bags, dim), dtype=indices.dtype, device=table.device) if want_max_indices else None
+    x = _ext(table, indices, odt, include_last_offset, psw, mi, stride, oob_flag)
+    lib.check(lib.dll.fwdmi_embedding_bag(_p(indices), _p(offsets), _p(dst), indices.numel(), n_bags, _p(table),
+                                          table.shape[0] if count is None else count, dim, data_offset, _op(mode),
+                                          C.byref(x), _stream(stream)))
+    return (out, mi) if want_max_indices else out
+
+
+def embedding_bag_fixed(table, indices, mode="sum", data_offset=0, out_dtype=None, oob_flag=None, stream=None):
+    """Fixed-length bags: ``indices`` is ``[B, L]`` -> ``[B, dim]``."""
+    table, indices = _dev(table, "table"), _dev(indices, "indices")
+    assert indices.dim() == 2
+    b, l = indices.shape
+    odt = table.dtype if out_dtype is None else out_dtype
+    out = torch.empty((b, table.shape[1]), dtype=odt, device=table.device)
+    x = _ext(table, indices, odt, oob_flag=oob_flag)
+    lib.check(lib.dll.fwdmi_embedding_bag_fixed(_p(indices), _p(out), b, l, _p(table), table.shape[0], table.shape[1],
+                                                data_offset, _op(mode), C.byref(x), _stream(stream)))
+    return out
+
+
+def gather(table, indices, data_offset=0, out_dtype=None, oob_flag=None, stream=None):
+    """Plain row gather: ``[B, L]`` ids -> ``[B, L, dim]``."""
+    table, indices = _dev(table, "table"), _dev(indices, "indices")
+    assert indices.dim() == 2
+    b, l = indices.shape
+    odt = table.dtype if out_dtype is None else out_dtype
+    out = torch.empty((b, l, table.shape[1]), dtype=odt, device=table.device)
+    x = _ext(table, indices, odt, oob_flag=oob_flag)
+    lib.check(lib.dll.fwdmi_gather(_p(indices), _p(out), b, l, _p(table), table.shape[0], table.shape[1],
+                                   data_offset, C.byref(x), _stream(stream)))
+    return out
+
+
+class MultiTableBatch:
+    """Device-resident descriptor array for ``fwdmi_embedding_bag_multi``.
+
+    Holds references to the tables / ids / offsets it points at so they stay alive.
+    """
+
+    def __init__(self, tables, indices, offsets, out_cols=None, data_offsets=None):
+        assert len(tables) == len(indices) == len(offsets) and tables
+        self.tables = [_dev(t, "table") for t in tables]
+        self.indices = [_dev(i, "indices") for i in indices]
+        self.offsets = [_dev(o, "offsets") for o in offsets]
+        self.dim = self.tables[0].shape[1]
+        self.n_bags = self.offsets[0].numel()
+        self.n_tables = len(tables)
+        out_cols = [t * self.dim for t in range(self.n_tables)] if out_cols is None else list(out_cols)
+        data_offsets = [0] * self.n_tables if data_offsets is None else list(data_offsets)
+        desc = np.zeros((self.n_tables, 7), np.int64)
+        for t in range(self.n_tables):
+            assert self.tables[t].shape[1] == self.dim and self.tables[t].dtype == self.tables[0].dtype
+            assert self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype
+            assert self.offsets[t].numel() == self.n_bags
+            desc[t] = (self.tables[t].data_ptr(), self.indices[t].data_ptr(), self.offsets[t].data_ptr(),
+                       self.tables[t].shape[0], self.indices[t].numel(), data_offsets[t], out_cols[t])
+        self.width = max(out_cols) + self.dim
+        self.total_indices = int(sum(i.numel() for i in self.indices))
+        self.desc = torch.from_numpy(desc).to(self.tables[0].device)
+
+    def forward(self, out=None, mode="sum", out_dtype=None, oob_flag=None, stream=None):
+        odt = self.tables[0].dtype if out_dtype is None else out_dtype
+        if out is None:
+            out = torch.empty((self.n_bags, self.width), dtype=odt, device=self.desc.device)
+        _dev(out, "out")
+        assert out.dtype == odt and out.shape[0] == self.n_bags and out.shape[1] >= self.width
+        x = _ext(self.tables[0], self.indices[0], odt, out_row_stride=out.shape[1], oob_flag=oob_flag)
+        avg = self.total_indices / max(1, self.n_bags * self.n_tables)
+        lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(self.desc), self.n_tables, self.n_bags, _p(out), self.dim,
+                                                    _op(mode), avg, C.byref(x), _stream(stream)))
+        return out
+
+
+def _params(gamma, beta, bias=None):
+    g, b = _dev(gamma, "gamma"), _dev(beta, "beta")
+    assert g.dtype == torch.float32 and b.dtype == torch.float32
+    if bias is not None:
+        assert _dev(bias, "bias").dtype == torch.float32
+    return g, b, bias
+
+
+def skip_layer_norm(x, gamma, beta, skip=None, bias=None, eps=0.0, out=None, stream=None):
+    """``LN(x (+ skip) (+ bias))`` over the last axis; gamma/beta/bias are fp32 device vectors."""
+    x = _dev(x, "input")
+    g, b, bias = _params(gamma, beta, bias)
+    ld = x.shape[-1]
+    assert g.numel() == ld and b.numel() == ld
+    if skip is not None:
+        assert _dev(skip, "skip").shape == x.shape and skip.dtype == x.dtype
+    out = torch.empty_like(x) if out is None else _dev(out, "out")
+    lib.check(lib.dll.fwdmi_skip_layer_norm(_stream(stream), ld, x.numel(), _p(x), _p(skip), _p(b), _p(g), _p(out),
+                                            _p(bias), _FDT[x.dtype], eps))
+    return out
+
+
+def layer_norm(x, gamma, beta, bias=None, eps=0.0, out=None, stream=None):
+    x = _dev(x, "input")
+    g, b, bias = _params(gamma, beta, bias)
+    ld = x.shape[-1]
+    out = torch.empty_like(x) if out is None else _dev(out, "out")
+    lib.check(lib.dll.fwdmi_layer_norm(_stream(stream), ld, x.numel(), _p(x), _p(b), _p(g), _p(out), _p(bias),
+                                       _FDT[x.dtype], eps))
+    return out
+
+
+def emb_layer_norm(input_ids, segment_ids, input_mask, word, pos, tok, gamma, beta, eps=0.0, oob_flag=None,
+                   out=None, mask_idx=None, stream=None):
+    """ids / mask are int32 ``[S, B]``; returns ``(out [S, B, H], mask_idx int32 [B])``."""
+    ids, seg = _dev(input_ids, "input_ids"), _dev(segment_ids, "segment_ids")
+    msk = _dev(input_mask, "input_mask") if input_mask is not None else None
+    assert ids.dtype == torch.int32 and seg.dtype == torch.int32 and ids.dim() == 2 and seg.shape == ids.shape
+    word, pos, tok = _dev(word, "word"), _dev(pos, "pos"), _dev(tok, "tok")
+    assert word.dtype == pos.dtype == tok.dtype
+    g, b, _ = _params(gamma, beta)
+    s, bsz = ids.shape
+    ld = word.shape[1]
+    if out is None:
+        out = torch.empty((s, bsz, ld), dtype=word.dtype, device=word.device)
+    if mask_idx is None and msk is not None:
+        mask_idx = torch.empty((bsz,), dtype=torch.int32, device=word.device)
+    lib.check(lib.dll.fwdmi_emb_layer_norm(_stream(stream), s, bsz, ld, _p(ids), _p(seg), _p(msk), _p(b), _p(g),
+                                           _p(word), _p(pos), _p(tok), word.shape[0], pos.shape[0], tok.shape[0],
+                                           _p(out), _p(mask_idx), _FDT[word.dtype], eps, _p(oob_flag)))
+    return out, mask_idx

@@ -1,0 +1,213 @@
+"""Python mirror of the plugin objects exported by ``libfwdmi.so``.
+
+Method names follow the reference's plugin interface (``getOutputDimensions``,
+``supportsFormatCombination``, ``configurePlugin``, ``enqueue``, ``serialize`` ... on plugins;
+``createPlugin`` / ``deserializePlugin`` / ``getFieldNames`` on creators;
+``getPluginCreator(name, version)`` on the registry), so host code and tests read like the
+reference's own layer creators.  Creator fields are given as numpy arrays / ints; ``enqueue``
+takes device tensors.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import lib
+
+_NP_FIELD = {np.dtype(np.float16): lib.FIELD_F16, np.dtype(np.float32): lib.FIELD_F32,
+             np.dtype(np.float64): lib.FIELD_F64, np.dtype(np.int8): lib.FIELD_I8,
+             np.dtype(np.int16): lib.FIELD_I16, np.dtype(np.int32): lib.FIELD_I32}
+_T2DT = {torch.float32: lib.F32, torch.float16: lib.F16, torch.int32: lib.I32, torch.int64: lib.I64,
+         torch.int8: lib.I8, torch.bool: lib.BOOL}
+_DT2T = {v: k for k, v in _T2DT.items()}
+
+
+class PluginFieldData:
+    """One creator field: a name plus a numpy array (scalars become 1-element int32 / float32)."""
+
+    def __init__(self, name, value, ftype=None):
+        if isinstance(value, (bool, int, np.integer)):
+            value = np.array([value], np.int32)
+        elif isinstance(value, float):
+            value = np.array([value], np.float32)
+        self.name = name
+        self.array = np.ascontiguousarray(value)
+        self.type = _NP_FIELD[self.array.dtype] if ftype is None else ftype
+
+    def c_field(self):
+        f = lib.PluginField()
+        f.name = self.name.encode()
+        f.data = self.array.ctypes.data
+        f.type = self.type
+        f.length = self.array.size
+        return f
+
+
+def _descs(items):
+    arr = (lib.TensorDesc * max(1, len(items)))()
+    for i, (shape, dtype) in enumerate(items):
+        arr[i] = lib.TensorDesc.of(shape, dtype)
+    return arr
+
+
+def _desc_of(t):
+    return (tuple(t.shape), _T2DT[t.dtype])
+
+
+class Plugin:
+    def __init__(self, handle):
+        if not handle:
+            raise lib.FwdmiError(lib.ERR_BAD_ARG, lib.last_error())
+        self._h = C.c_void_p(handle)
+
+    # -- shape / format negotiation ---------------------------------------------------------
+    def getNbOutputs(self):
+        return lib.dll.fwdmi_plugin_get_nb_outputs(self._h)
+
+    def getOutputDimensions(self, outputIndex, inputs):
+        arr = (lib.Dims * max(1, len(inputs)))(*[lib.Dims.of(*s) for s in inputs])
+        out = lib.Dims()
+        lib.check(lib.dll.fwdmi_plugin_get_output_dimensions(self._h, outputIndex, arr, len(inputs), C.byref(out)))
+        return out.tolist()
+
+    def supportsFormatCombination(self, pos, inOut, nbInputs, nbOutputs):
+        """``inOut``: list of (shape, dtype[, format])."""
+        arr = (lib.TensorDesc * max(1, len(inOut)))()
+        for i, it in enumerate(inOut):
+            arr[i] = lib.TensorDesc.of(it[0], it[1], it[2] if len(it) > 2 else lib.FORMAT_LINEAR)
+        rc = lib.dll.fwdmi_plugin_supports_format_combination(self._h, pos, arr, nbInputs, nbOutputs)
+        if rc < 0:
+            raise lib.FwdmiError(rc, "supportsFormatCombination: bad arguments")
+        return bool(rc)
+
+    def getOutputDataType(self, index, inputTypes):
+        arr = (C.c_int32 * max(1, len(inputTypes)))(*inputTypes)
+        return lib.dll.fwdmi_plugin_get_output_data_type(self._h, index, arr, len(inputTypes))
+
+    # -- lifecycle ------------------------------------------------------------------------------
+    def configurePlugin(self, inputs, outputs):
+        """``inputs`` / ``outputs``: lists of (shape, dtype).  Uploads tables to the current device."""
+        lib.check(lib.dll.fwdmi_plugin_configure(self._h, _descs(inputs), len(inputs), _descs(outputs), len(outputs)))
+
+    def getWorkspaceSize(self, inputs, outputs):
+        return lib.dll.fwdmi_plugin_get_workspace_size(self._h, _descs(inputs), len(inputs), _descs(outputs),
+                                                       len(outputs))
+
+    def initialize(self):
+        return lib.dll.fwdmi_plugin_initialize(self._h)
+
+    def terminate(self):
+        lib.dll.fwdmi_plugin_terminate(self._h)
+
+    def enqueue_raw(self, in_descs, out_descs, in_ptrs, out_ptrs, stream_handle=None):
+        """``enqueue`` on raw device addresses; returns the status instead of raising."""
+        ins = (C.c_void_p * max(1, len(in_ptrs)))(*in_ptrs)
+        outs = (C.c_void_p * max(1, len(out_ptrs)))(*out_ptrs)
+        s = torch.cuda.current_stream().cuda_stream if stream_handle is None else stream_handle
+        return lib.dll.fwdmi_plugin_enqueue(self._h, _descs(in_descs), _descs(out_descs), ins, outs, None,
+                                            C.c_void_p(s))
+
+    def enqueue(self, inputs, outputs, stream=None):
+        """Device tensors in, device tensors out (written in place); raises on a non-zero status."""
+        for t in list(inputs) + list(outputs):
+            if not t.is_cuda or not t.is_contiguous():
+                raise RuntimeError("enqueue needs contiguous device tensors")
+        s = None if stream is None else stream.cuda_stream
+        rc = self.enqueue_raw([_desc_of(t) for t in inputs], [_desc_of(t) for t in outputs],
+                              [t.data_ptr() for t in inputs], [t.data_ptr() for t in outputs], s)
+        return lib.check(rc)
+
+    def __call__(self, *inputs):
+        """Convenience: infer output shapes/types, allocate, enqueue, return the outputs."""
+        shapes = [tuple(t.shape) for t in inputs]
+        outs = []
+        for i in range(self.getNbOutputs()):
+            dims = self.getOutputDimensions(i, shapes)
+            dt = self.getOutputDataType(i, [_T2DT[t.dtype] for t in inputs])
+            outs.append(torch.empty(dims, dtype=_DT2T[dt], device=inputs[0].device))
+        self.configurePlugin([_desc_of(t) for t in inputs], [_desc_of(t) for t in outs])
+        self.enqueue(list(inputs), outs)
+        return outs[0] if len(outs) == 1 else tuple(outs)
+
+    # -- identity / persistence -----------------------------------------------------------------
+    def getSerializationSize(self):
+        return lib.dll.fwdmi_plugin_get_serialization_size(self._h)
+
+    def serialize(self):
+        buf = np.zeros(self.getSerializationSize(), np.uint8)
+        lib.check(lib.dll.fwdmi_plugin_serialize(self._h, C.c_void_p(buf.ctypes.data)))
+        return buf.tobytes()
+
+    def getPluginType(self):
+        return lib.dll.fwdmi_plugin_get_type(self._h).decode()
+
+    def getPluginVersion(self):
+        return lib.dll.fwdmi_plugin_get_version(self._h).decode()
+
+    def setPluginNamespace(self, ns):
+        self._ns = ns.encode()  # the reference borrows the pointer; keep it alive anyway
+        lib.dll.fwdmi_plugin_set_namespace(self._h, self._ns)
+
+    def getPluginNamespace(self):
+        return lib.dll.fwdmi_plugin_get_namespace(self._h).decode()
+
+    def clone(self):
+        return Plugin(lib.dll.fwdmi_plugin_clone(self._h))
+
+    def takeOobFlag(self):
+        rc = lib.dll.fwdmi_plugin_take_oob_flag(self._h, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        if rc < 0:
+            raise lib.FwdmiError(rc, lib.last_error())
+        return bool(rc)
+
+    def destroy(self):
+        if self._h:
+            lib.dll.fwdmi_plugin_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class PluginCreator:
+    def __init__(self, handle):
+        self._h = C.c_void_p(handle)
+
+    def getPluginName(self):
+        return lib.dll.fwdmi_creator_name(self._h).decode()
+
+    def getPluginVersion(self):
+        return lib.dll.fwdmi_creator_version(self._h).decode()
+
+    def getFieldNames(self):
+        n = lib.dll.fwdmi_creator_num_fields(self._h)
+        return [(lib.dll.fwdmi_creator_field_name(self._h, i).decode(), lib.dll.fwdmi_creator_field_type(self._h, i))
+                for i in range(n)]
+
+    def createPlugin(self, name, fields):
+        """``fields``: list of PluginFieldData (or (name, value) pairs).  Raises FwdmiError on a
+        contract violation (where the reference aborts)."""
+        fields = [f if isinstance(f, PluginFieldData) else PluginFieldData(*f) for f in fields]
+        arr = (lib.PluginField * max(1, len(fields)))(*[f.c_field() for f in fields])
+        return Plugin(lib.dll.fwdmi_creator_create_plugin(self._h, name.encode(), arr, len(fields)))
+
+    def deserializePlugin(self, name, data):
+        buf = np.frombuffer(bytes(data), np.uint8)
+        ptr = C.c_void_p(buf.ctypes.data) if buf.size else C.c_void_p(0)
+        return Plugin(lib.dll.fwdmi_creator_deserialize_plugin(self._h, name.encode(), ptr, buf.size))
+
+
+class PluginRegistry:
+    def getPluginCreator(self, name, version):
+        h = lib.dll.fwdmi_get_plugin_creator(name.encode(), version.encode())
+        return PluginCreator(h) if h else None
+
+    def getPluginCreatorList(self):
+        return [PluginCreator(lib.dll.fwdmi_registry_at(i)) for i in range(lib.dll.fwdmi_registry_size())]
+
+
+def getPluginRegistry():
+    return PluginRegistry()

@@ -1,0 +1,259 @@
+/*
+ * fwdmi.h -- C ABI of the MI355X (gfx950) embedding-side plugin path.
+ *
+ * Two layers are exported from libfwdmi.so, both `extern "C"`, plain pointers and sizes only:
+ *
+ *  1. kernel launchers: one per kernel family, the functions a plugin's enqueue() calls.  They
+ *     take DEVICE pointers, enqueue work on the given HIP stream and return without
+ *     synchronising or allocating.
+ *  2. plugin objects: an opaque-handle view of the C++ plugin classes (creator lookup, field
+ *     parsing, shape inference, format negotiation, configure, enqueue, serialize, clone) for
+ *     hosts that cannot include the C++ header (Python ctypes, cgo, JNI).
+ *
+ * Every function returns an int status unless noted: 0 ok, negative on error (never aborts).
+ * Paths in "replaces" notes are relative to the reference tree (Tencent/Forward).
+ */
+#ifndef FWDMI_H_
+#define FWDMI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes ---------------------------------------------------------------------- */
+#define FWDMI_OK 0
+#define FWDMI_ERR_UNSUPPORTED (-1) /* dtype / format the path does not handle (reference: enqueue returns -1,
+                                      embedding_bag_plugin.cpp:182-185) */
+#define FWDMI_ERR_BAD_ARG (-2)     /* null pointer, negative size, shape mismatch */
+#define FWDMI_ERR_HIP (-3)         /* a HIP runtime call failed; fwdmi_last_error() has the text */
+#define FWDMI_ERR_NOT_CONFIGURED (-4)
+#define FWDMI_ERR_TRUNCATED (-5)   /* serialized blob shorter than its own header says */
+
+/* ---- element types: values follow nvinfer1::DataType; I64 is an extension ---------------- */
+#define FWDMI_F32 0
+#define FWDMI_F16 1
+#define FWDMI_I8 2
+#define FWDMI_I32 3
+#define FWDMI_BOOL 4
+#define FWDMI_I64 10
+
+/* ---- plugin field types: values follow nvinfer1::PluginFieldType -------------------------- */
+#define FWDMI_FIELD_F16 0
+#define FWDMI_FIELD_F32 1
+#define FWDMI_FIELD_F64 2
+#define FWDMI_FIELD_I8 3
+#define FWDMI_FIELD_I16 4
+#define FWDMI_FIELD_I32 5
+#define FWDMI_FIELD_CHAR 6
+#define FWDMI_FIELD_DIMS 7
+#define FWDMI_FIELD_UNKNOWN 8
+
+/* ---- tensor format: nvinfer1::TensorFormat::kLINEAR ---------------------------------------- */
+#define FWDMI_FORMAT_LINEAR 0
+
+/* ---- bag reduction codes: ReduceOperation, embedding_bag_plugin.h:39 ----------------------- */
+#define FWDMI_OP_SUM 0
+#define FWDMI_OP_MEAN 1
+#define FWDMI_OP_MAX 2
+#define FWDMI_OP_SQUARE_SUM 3
+#define FWDMI_OP_GATHER 999
+
+const char* fwdmi_version(void);
+/* Text of the most recent failure on the calling thread ("" if none). */
+const char* fwdmi_last_error(void);
+/* Number of HIP devices visible (0 without a GPU; never an error). */
+int fwdmi_device_count(void);
+
+/* ========================================================================================= *
+ *  1. Kernel launchers
+ * ========================================================================================= */
+
+/*
+ * Options beyond what the reference launchers take.  NULL means the reference's contract:
+ * fp32 table, int32 indices, fp32 output rows packed at stride `dim`.
+ */
+typedef struct fwdmi_bag_ext {
+  int32_t table_dtype;         /* FWDMI_F32 | FWDMI_F16 */
+  int32_t index_dtype;         /* FWDMI_I32 | FWDMI_I64 (indices, offsets, max_indices) */
+  int32_t out_dtype;           /* FWDMI_F32 | FWDMI_F16 */
+  int32_t include_last_offset; /* offsets has n_bags+1 entries */
+  const void* per_sample_weights; /* device, table dtype, [n_indices]; SUM only; may be NULL */
+  void* max_indices;           /* device, index dtype, [n_bags, dim]; MAX only; may be NULL */
+  int64_t out_row_stride;      /* elements between output rows; 0 = dim (lets several tables
+                                  write column blocks of one concatenated matrix) */
+  int32_t* oob_flag;           /* device int, set to 1 (sticky) when an id falls outside
+                                  [data_offset, data_offset+count); may be NULL */
+} fwdmi_bag_ext;
+
+/*
+ * Variable-length bags: bag b = input[input_2[b] .. input_2[b+1]), last bag ends at input_size.
+ * replaces EmbeddingBag(), embedding_bag_plugin.h:47-49 / embedding_bag_plugin.cu:198-206.
+ *   input    [input_size] ids          input_2 [block_size] offsets (block_size = number of bags)
+ *   output   [block_size, dim]         data    [count, dim] table, row-major
+ * Ids outside [data_offset, data_offset+count) are skipped (embedding_bag_plugin.cu:94).
+ * op_type MEAN divides by the bag length, MAX keeps the first maximum; empty bags give zeros.
+ */
+int fwdmi_embedding_bag(const void* input, const void* input_2, void* output, int64_t input_size,
+                        int64_t block_size, const void* data, int64_t count, int32_t dim,
+                        int64_t data_offset, int32_t op_type, const fwdmi_bag_ext* ext, void* stream);
+
+/*
+ * Fixed-length bags: input is [batch_size, offset] ids, bag b = row b.
+ * replaces EmbeddingBagWithFixedOffset(), embedding_bag_plugin.h:43-45 / .cu:190-196.
+ */
+int fwdmi_embedding_bag_fixed(const void* input, void* output, int64_t batch_size, int64_t offset,
+                              const void* data, int64_t count, int32_t dim, int64_t data_offset,
+                              int32_t op_type, const fwdmi_bag_ext* ext, void* stream);
+
+/*
+ * Plain row gather (op 999): output[i, :] = data[input[i] - data_offset, :] for the
+ * batch_size*offset ids; out-of-range ids produce zero rows.
+ * replaces Gather(), embedding_bag_plugin.h:40-41 / .cu:182-188.
+ */
+int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t offset,
+                 const void* data, int64_t count, int32_t dim, int64_t data_offset,
+                 const fwdmi_bag_ext* ext, void* stream);
+
+/*
+ * One table of a multi-table batch.  The array of these lives in DEVICE memory.
+ */
+typedef struct fwdmi_bag_table {
+  const void* data;    /* [count, dim], 16-byte aligned */
+  const void* input;   /* [input_size] ids */
+  const void* input_2; /* [n_bags] offsets (+1 with include_last_offset) */
+  int64_t count;
+  int64_t input_size;
+  int64_t data_offset;
+  int64_t out_col;     /* first output column of this table's block (a multiple of 8) */
+} fwdmi_bag_table;
+
+/*
+ * All tables of a DLRM-style sparse stage in one launch: every table reduces the same number
+ * of bags with the same dim / dtypes and writes its [n_bags, dim] block at column out_col of
+ * one [n_bags, out_row_stride] matrix.  Equivalent to n_tables calls of fwdmi_embedding_bag
+ * with ext->out_row_stride set (the reference issues one plugin enqueue per table,
+ * embedding_bag_plugin.cpp:146-189, and concatenates afterwards).
+ * `avg_bag_len` (>0) is a sizing hint: the mean ids per bag over the batch.
+ * Per-sample weights and max_indices are not available in this form.
+ */
+int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_tables, int64_t n_bags,
+                              void* output, int32_t dim, int32_t op_type, double avg_bag_len,
+                              const fwdmi_bag_ext* ext, void* stream);
+
+/*
+ * out = gamma * (x - mean) * rsqrt(var + eps) + beta,  x = input (+ bias), per row of ld.
+ * n = total elements (rows = n / ld).  gamma/beta/bias: device fp32 [ld]; bias may be NULL.
+ * dtype: FWDMI_F32 | FWDMI_F16 for input and output.  The reference has no eps (pass 0).
+ * replaces computeLayerNorm<T,hasBias>(), layer_norm_plugin.h:37-39 / layer_norm_kernel.cu:278-305.
+ */
+int fwdmi_layer_norm(void* stream, int32_t ld, int64_t n, const void* input, const float* beta,
+                     const float* gamma, void* output, const float* bias, int32_t dtype, float eps);
+
+/*
+ * out = LN(input + skip (+ bias)): the arithmetic of "CustomSkipLayerNormPluginDynamic" v1 as
+ * the reference wires it (trt_bert_creator.h:199-239, inputs {input, skip}).
+ */
+int fwdmi_skip_layer_norm(void* stream, int32_t ld, int64_t n, const void* input, const void* skip,
+                          const float* beta, const float* gamma, void* output, const float* bias,
+                          int32_t dtype, float eps);
+
+/*
+ * BERT embedding lookup fused with LayerNorm: the arithmetic of
+ * "CustomEmbLayerNormPluginDynamic" v1 as the reference wires it (trt_bert_creator.h:113-155).
+ *   input_ids, segment_ids, input_mask : int32 [S, B]   (token t = s*B + b)
+ *   word [word_count, ld], pos [pos_count, ld], tok [tok_count, ld] in `dtype`
+ *   output [S, B, ld] in `dtype`;  mask_idx int32 [B] = first s with input_mask[s,b]==0, else S
+ *   (mask_idx / input_mask may both be NULL).  Out-of-table ids add a zero row and raise
+ *   *oob_flag (may be NULL).
+ */
+int fwdmi_emb_layer_norm(void* stream, int32_t S, int32_t B, int32_t ld, const int32_t* input_ids,
+                         const int32_t* segment_ids, const int32_t* input_mask, const float* beta,
+                         const float* gamma, const void* word, const void* pos, const void* tok,
+                         int32_t word_count, int32_t pos_count, int32_t tok_count, void* output,
+                         int32_t* mask_idx, int32_t dtype, float eps, int32_t* oob_flag);
+
+/* ========================================================================================= *
+ *  2. Plugin objects (opaque handles over the C++ classes in fwdmi_plugin.h)
+ * ========================================================================================= */
+
+typedef struct fwdmi_plugin fwdmi_plugin;   /* an IPluginV2DynamicExt */
+typedef struct fwdmi_creator fwdmi_creator; /* an IPluginCreator (owned by the registry) */
+
+typedef struct fwdmi_dims {
+  int32_t nbDims;
+  int32_t d[8];
+} fwdmi_dims; /* nvinfer1::Dims */
+
+typedef struct fwdmi_tensor_desc {
+  fwdmi_dims dims;
+  int32_t type;   /* FWDMI_F32 ... */
+  int32_t format; /* FWDMI_FORMAT_LINEAR */
+  float scale;
+} fwdmi_tensor_desc; /* nvinfer1::PluginTensorDesc */
+
+typedef struct fwdmi_plugin_field {
+  const char* name;
+  const void* data; /* borrowed: the plugin copies what it keeps */
+  int32_t type;     /* FWDMI_FIELD_* */
+  int32_t length;   /* element count */
+} fwdmi_plugin_field; /* nvinfer1::PluginField */
+
+/* getPluginRegistry()->getPluginCreator(name, version), trt_embedding_bag_creator.h:54-55.
+ * Registered: "EmbeddingBag_TRT"/"001", "CustomEmbLayerNormPluginDynamic"/"1",
+ * "CustomSkipLayerNormPluginDynamic"/"1", "ForwardLayerNormPluginDynamic"/"1". NULL if absent. */
+fwdmi_creator* fwdmi_get_plugin_creator(const char* name, const char* version);
+int fwdmi_registry_size(void);
+fwdmi_creator* fwdmi_registry_at(int i);
+
+const char* fwdmi_creator_name(fwdmi_creator* c);
+const char* fwdmi_creator_version(fwdmi_creator* c);
+int fwdmi_creator_num_fields(fwdmi_creator* c);
+/* name / type of declared field i (IPluginCreator::getFieldNames). */
+const char* fwdmi_creator_field_name(fwdmi_creator* c, int i);
+int fwdmi_creator_field_type(fwdmi_creator* c, int i);
+/* IPluginCreator::createPlugin; NULL on a contract violation (fwdmi_last_error says which). */
+fwdmi_plugin* fwdmi_creator_create_plugin(fwdmi_creator* c, const char* name,
+                                          const fwdmi_plugin_field* fields, int n_fields);
+/* IPluginCreator::deserializePlugin; NULL on a truncated / malformed blob. */
+fwdmi_plugin* fwdmi_creator_deserialize_plugin(fwdmi_creator* c, const char* name, const void* data,
+                                               size_t length);
+
+int fwdmi_plugin_get_nb_outputs(fwdmi_plugin* p);
+/* getOutputDimensions on concrete dims; writes *out. */
+int fwdmi_plugin_get_output_dimensions(fwdmi_plugin* p, int output_index, const fwdmi_dims* inputs,
+                                       int nb_inputs, fwdmi_dims* out);
+/* 1 supported, 0 not, negative on bad arguments. */
+int fwdmi_plugin_supports_format_combination(fwdmi_plugin* p, int pos, const fwdmi_tensor_desc* in_out,
+                                             int nb_inputs, int nb_outputs);
+/* configurePlugin: uploads tables / parameters to the current device (needs a GPU). */
+int fwdmi_plugin_configure(fwdmi_plugin* p, const fwdmi_tensor_desc* in, int nb_inputs,
+                           const fwdmi_tensor_desc* out, int nb_outputs);
+size_t fwdmi_plugin_get_workspace_size(fwdmi_plugin* p, const fwdmi_tensor_desc* in, int nb_inputs,
+                                       const fwdmi_tensor_desc* out, int nb_outputs);
+int fwdmi_plugin_initialize(fwdmi_plugin* p);
+void fwdmi_plugin_terminate(fwdmi_plugin* p);
+/* enqueue: device pointers, stream-ordered, no host sync, no allocation. */
+int fwdmi_plugin_enqueue(fwdmi_plugin* p, const fwdmi_tensor_desc* in_desc,
+                         const fwdmi_tensor_desc* out_desc, const void* const* inputs,
+                         void* const* outputs, void* workspace, void* stream);
+size_t fwdmi_plugin_get_serialization_size(fwdmi_plugin* p);
+int fwdmi_plugin_serialize(fwdmi_plugin* p, void* buffer);
+const char* fwdmi_plugin_get_type(fwdmi_plugin* p);
+const char* fwdmi_plugin_get_version(fwdmi_plugin* p);
+void fwdmi_plugin_set_namespace(fwdmi_plugin* p, const char* ns);
+const char* fwdmi_plugin_get_namespace(fwdmi_plugin* p);
+int fwdmi_plugin_get_output_data_type(fwdmi_plugin* p, int index, const int32_t* input_types,
+                                      int nb_inputs);
+fwdmi_plugin* fwdmi_plugin_clone(fwdmi_plugin* p);
+void fwdmi_plugin_destroy(fwdmi_plugin* p);
+/* Reads and clears the plugin's sticky "an id was out of range" device flag (synchronises the
+ * stream; diagnostic, not part of the reference contract). Returns 0/1 or a negative status. */
+int fwdmi_plugin_take_oob_flag(fwdmi_plugin* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FWDMI_H_ */

@@ -1,0 +1,51 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/fwdmi.h declares."""
+import re
+import subprocess
+
+from forward_amd import lib
+
+
+def declared_symbols():
+    text = open(lib.HEADER_PATH).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b(fwdmi_[a-z0-9_]+)\s*\(", text))
+
+
+def test_header_matches_binding_table():
+    assert declared_symbols() == set(lib.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    out = subprocess.check_output(["nm", "-D", "--defined-only", lib.LIB_PATH], text=True)
+    exported = {l.split()[-1] for l in out.splitlines() if " T " in l}
+    missing = declared_symbols() - exported
+    assert not missing, missing
+    extra = {s for s in exported if s.startswith("fwdmi_")} - declared_symbols()
+    assert not extra, extra
+
+
+def test_basic_calls_without_gpu():
+    assert lib.dll.fwdmi_version().startswith(b"fwdmi")
+    assert lib.dll.fwdmi_device_count() >= 0
+    assert lib.dll.fwdmi_registry_size() == 5
+
+
+def test_launchers_validate_before_touching_the_gpu():
+    import ctypes as C
+    x = lib.BagExt()
+    x.table_dtype, x.index_dtype, x.out_dtype = lib.I8, lib.I32, lib.F32
+    rc = lib.dll.fwdmi_embedding_bag(None, None, None, 0, 4, None, 10, 8, 0, 0, C.byref(x), None)
+    assert rc == lib.ERR_UNSUPPORTED and "dtype" in lib.last_error()
+    rc = lib.dll.fwdmi_embedding_bag(None, None, None, 0, 4, None, 10, 8, 0, 7, None, None)
+    assert rc == lib.ERR_UNSUPPORTED
+    rc = lib.dll.fwdmi_embedding_bag(None, None, None, 0, 4, None, 10, 8, 0, 0, None, None)
+    assert rc == lib.ERR_BAD_ARG                       # null output
+    rc = lib.dll.fwdmi_embedding_bag(None, None, None, 0, 0, None, 10, 8, 0, 0, None, None)
+    assert rc == lib.OK                                # zero bags: nothing to do
+    rc = lib.dll.fwdmi_layer_norm(None, 10, 25, None, None, None, None, None, lib.F32, 0.0)
+    assert rc == lib.ERR_BAD_ARG and "multiple" in lib.last_error()
+    rc = lib.dll.fwdmi_layer_norm(None, 10, 20, None, None, None, None, None, lib.I8, 0.0)
+    assert rc == lib.ERR_UNSUPPORTED
+    rc = lib.dll.fwdmi_emb_layer_norm(None, 4, 2, 8, None, None, None, None, None, None, None, None, 1, 1, 1, None,
+                                      None, lib.F16, 0.0, None)
+    assert rc == lib.ERR_BAD_ARG

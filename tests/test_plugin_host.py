@@ -1,0 +1,219 @@
+"""Host-side plugin contract: registry, creator fields, shape / format rules, serialized bytes,
+clone, error statuses.  Everything here runs without a GPU (no configure / enqueue)."""
+import struct
+
+import numpy as np
+import pytest
+
+from forward_amd import lib, plugin
+from forward_amd.plugin import PluginFieldData as F
+
+REG = plugin.getPluginRegistry()
+
+
+def bag_fields(table, op=0, offset=0):
+    count, dim = table.shape
+    # order and types of trt_embedding_bag_creator.h:56-65
+    return [F("dim", dim), F("count", count), F("offset", offset), F("op", op), F("data", table)]
+
+
+def test_registry_lookup():
+    names = {(c.getPluginName(), c.getPluginVersion()) for c in REG.getPluginCreatorList()}
+    assert names == {("EmbeddingBag_TRT", "001"), ("EmbeddingBag_TRT", "002"),
+                     ("ForwardLayerNormPluginDynamic", "1"), ("CustomSkipLayerNormPluginDynamic", "1"),
+                     ("CustomEmbLayerNormPluginDynamic", "1")}
+    assert REG.getPluginCreator("EmbeddingBag_TRT", "003") is None
+    assert REG.getPluginCreator("Nope", "1") is None
+
+
+def test_embedding_bag_creator_fields():
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    assert c.getFieldNames() == [("dim", lib.FIELD_I32), ("count", lib.FIELD_I32), ("offset", lib.FIELD_I32),
+                                 ("op", lib.FIELD_I32), ("data", lib.FIELD_F32)]
+    table = np.arange(20, dtype=np.float32).reshape(5, 4)
+    p = c.createPlugin("embedding_bag", bag_fields(table))
+    assert p.getPluginType() == "EmbeddingBag_TRT" and p.getPluginVersion() == "001"
+    assert p.getNbOutputs() == 1 and p.getPluginNamespace() == ""
+    assert p.getWorkspaceSize([((5,), lib.I32), ((5,), lib.I32)], [((5, 4), lib.F32)]) == 0
+    # contract violations: wrong field count, unknown name, wrong type (the reference aborts)
+    with pytest.raises(lib.FwdmiError, match="expected 5 fields"):
+        c.createPlugin("x", bag_fields(table)[:4])
+    with pytest.raises(lib.FwdmiError, match="unknown field"):
+        c.createPlugin("x", bag_fields(table)[:4] + [F("weights", table)])
+    with pytest.raises(lib.FwdmiError, match="INT32"):
+        c.createPlugin("x", [F("dim", np.array([4.0], np.float32))] + bag_fields(table)[1:])
+    with pytest.raises(lib.FwdmiError, match="FLOAT32"):
+        c.createPlugin("x", bag_fields(table)[:4] + [F("data", table.astype(np.float16))])
+    with pytest.raises(lib.FwdmiError, match="dim\\*count"):
+        c.createPlugin("x", bag_fields(table)[:4] + [F("data", table[:3])])
+
+
+def test_embedding_bag_output_dimensions_and_formats():
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    table = np.zeros((50, 16), np.float32)
+    p = c.createPlugin("embedding_bag", bag_fields(table, op=0))
+    assert p.getOutputDimensions(0, [(10, 5)]) == [10, 16]                  # fixed-length bags
+    assert p.getOutputDimensions(0, [(1056,), (64,)]) == [64, 16]           # ids + offsets
+    assert p.getOutputDimensions(0, [(1056,), (1, 64)]) == [64, 16]         # offsets selected from a [1,B] slice
+    with pytest.raises(lib.FwdmiError):
+        p.getOutputDimensions(0, [(1056,)])                                 # single input must be 2-D
+    with pytest.raises(lib.FwdmiError):
+        p.getOutputDimensions(0, [(1056,), (2, 64)])
+    with pytest.raises(lib.FwdmiError):
+        p.getOutputDimensions(1, [(10, 5)])
+    g = c.createPlugin("gather", bag_fields(table, op=999))
+    assert g.getOutputDimensions(0, [(1, 10)]) == [1, 10, 16]
+    with pytest.raises(lib.FwdmiError, match="GATHER"):
+        g.getOutputDimensions(0, [(10,), (2,)])
+    g1 = c.createPlugin("gather", bag_fields(np.zeros((50, 1), np.float32), op=999))
+    assert g1.getOutputDimensions(0, [(1, 3)]) == [1, 3]                    # dim == 1 keeps the input shape
+
+    io = [((100,), lib.I32), ((8,), lib.I32), ((8, 16), lib.F32)]
+    assert all(p.supportsFormatCombination(i, io, 2, 1) for i in range(3))
+    assert not p.supportsFormatCombination(0, [((100,), lib.I64)] + io[1:], 2, 1)
+    assert not p.supportsFormatCombination(2, io[:2] + [((8, 16), lib.F16)], 2, 1)
+    assert not p.supportsFormatCombination(0, [((100,), lib.I32, 1)] + io[1:], 2, 1)   # non-linear format
+    assert not p.supportsFormatCombination(0, io + io, 3, 1)                          # at most two inputs
+    assert p.getOutputDataType(0, [lib.I32, lib.I32]) == lib.F32
+
+
+def test_embedding_bag_serialization_layout_and_roundtrip():
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    table = np.random.default_rng(0).standard_normal((7, 3)).astype(np.float32)
+    p = c.createPlugin("embedding_bag", bag_fields(table, op=3, offset=11))
+    blob = p.serialize()
+    # int dim | int count | int data_offset | int op | size_t n | float[n]   (embedding_bag_plugin.cpp:191-202)
+    assert len(blob) == p.getSerializationSize() == 24 + 4 * 21
+    assert struct.unpack("<iiiiQ", blob[:24]) == (3, 7, 11, 3, 21)
+    assert blob[24:] == table.tobytes()
+    q = c.deserializePlugin("embedding_bag", blob)
+    assert q.serialize() == blob
+    assert q.clone().serialize() == blob
+    for cut in (0, 3, 23, 24, len(blob) - 1):
+        with pytest.raises(lib.FwdmiError):
+            c.deserializePlugin("embedding_bag", blob[:cut])
+    bad = bytearray(blob)
+    bad[0:4] = struct.pack("<i", 4)                                          # dim no longer matches n
+    with pytest.raises(lib.FwdmiError, match="inconsistent"):
+        c.deserializePlugin("embedding_bag", bytes(bad))
+
+
+def test_embedding_bag_extended_version():
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "002")
+    table = np.random.default_rng(1).standard_normal((9, 8)).astype(np.float16)
+    p = c.createPlugin("embedding_bag", bag_fields(table) + [F("index_type", lib.I64), F("output_fp16", 1),
+                                                            F("include_last_offset", 1), F("per_sample_weights", 1)])
+    assert p.getPluginVersion() == "002"
+    assert p.getOutputDimensions(0, [(40,), (5,), (40,)]) == [4, 8]          # include_last_offset: B+1 offsets
+    io = [((40,), lib.I64), ((5,), lib.I64), ((40,), lib.F16), ((4, 8), lib.F16)]
+    assert all(p.supportsFormatCombination(i, io, 3, 1) for i in range(4))
+    assert not p.supportsFormatCombination(0, [((40,), lib.I32)] + io[1:], 3, 1)
+    assert p.getOutputDataType(0, [lib.I64, lib.I64, lib.F16]) == lib.F16
+    blob = p.serialize()
+    assert struct.unpack("<9iQ", blob[:44]) == (8, 9, 0, 0, lib.F16, lib.I64, lib.F16, 1, 1, 72)
+    assert blob[44:] == table.tobytes()
+    assert c.deserializePlugin("e", blob).serialize() == blob
+    with pytest.raises(lib.FwdmiError, match="SUM"):
+        c.createPlugin("e", bag_fields(table, op=2) + [F("per_sample_weights", 1)])
+    # the five reference fields alone are accepted by the extended creator too
+    assert c.createPlugin("e", bag_fields(table.astype(np.float32))).getOutputDataType(0, [lib.I32]) == lib.F32
+
+
+def test_enqueue_before_configure_and_wrong_dtype():
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    p = c.createPlugin("embedding_bag", bag_fields(np.zeros((5, 4), np.float32)))
+    rc = p.enqueue_raw([((5,), lib.I32), ((5,), lib.I32)], [((5, 4), lib.F32)], [0, 0], [0], stream_handle=0)
+    assert rc == lib.ERR_NOT_CONFIGURED
+    p.terminate()            # harmless before configure
+    p.setPluginNamespace("ns")
+    assert p.getPluginNamespace() == "ns" and p.clone().getPluginNamespace() == "ns"
+
+
+def ln_fields(ld, type_id, rng, bias=False, extra=()):
+    # order of trt_normalization_creator.h:147-157 (ld, beta, gamma, type_id, has_skip, batch_size)
+    f = [F("ld", ld), F("beta", rng.standard_normal(ld).astype(np.float32)),
+         F("gamma", rng.standard_normal(ld).astype(np.float32)), F("type_id", type_id)]
+    if bias:
+        f.append(F("bias", rng.standard_normal(ld).astype(np.float32)))
+    return f + list(extra)
+
+
+@pytest.mark.parametrize("name,n_in", [("ForwardLayerNormPluginDynamic", 1), ("CustomSkipLayerNormPluginDynamic", 2)])
+def test_layer_norm_plugins_host_contract(name, n_in):
+    rng = np.random.default_rng(2)
+    c = REG.getPluginCreator(name, "1")
+    assert [n for n, _ in c.getFieldNames()][:5] == ["ld", "type_id", "beta", "gamma", "bias"]
+    fields = ln_fields(10, lib.F32, rng, extra=[F("has_skip", 0), F("batch_size", 16)])   # unknown fields ignored
+    p = c.createPlugin("skip_layer_norm", fields)
+    assert p.getPluginType() == name and p.getPluginVersion() == "1" and p.getNbOutputs() == 1
+    shapes = [(20, 5, 10)] * n_in
+    assert p.getOutputDimensions(0, shapes) == [20, 5, 10]
+    with pytest.raises(lib.FwdmiError):
+        p.getOutputDimensions(0, shapes + [(20, 5, 10)])
+    io = [((20, 5, 10), lib.F32)] * (n_in + 1)
+    assert all(p.supportsFormatCombination(i, io, n_in, 1) for i in range(n_in + 1))
+    assert not p.supportsFormatCombination(0, [((20, 5, 10), lib.F16)] * (n_in + 1), n_in, 1)
+    assert not p.supportsFormatCombination(n_in, io[:-1] + [((20, 5, 10), lib.F16)], n_in, 1)
+    assert p.getOutputDataType(0, [lib.F32] * n_in) == lib.F32
+    # DataType mType | DataType mCfgType | size_t mLd | bool mHasBias | beta | gamma   (layer_norm_plugin.cpp:257-277)
+    blob = p.serialize()
+    assert len(blob) == p.getSerializationSize() == 4 + 4 + 8 + 1 + 2 * 10 * 4
+    assert struct.unpack("<iiQ?", blob[:17]) == (lib.F32, lib.F32, 10, False)
+    assert blob[17:57] == fields[1].array.tobytes() and blob[57:97] == fields[2].array.tobytes()
+    assert c.deserializePlugin("x", blob).serialize() == blob
+    assert p.clone().serialize() == blob
+    for cut in (0, 16, 17, 96):
+        with pytest.raises(lib.FwdmiError):
+            c.deserializePlugin("x", blob[:cut])
+
+    # half precision: parameters are stored (and serialized) as fp16; bias and eps extend the blob
+    f16 = ln_fields(8, lib.F16, rng, bias=True, extra=[F("eps", np.array([1e-12], np.float32))])
+    h = c.createPlugin("ln", f16)
+    blob = h.serialize()
+    assert len(blob) == 17 + 3 * 8 * 2 + 4
+    assert struct.unpack("<iiQ?", blob[:17]) == (lib.F16, lib.F16, 8, True)
+    assert blob[17:33] == f16[1].array.astype(np.float16).tobytes()
+    assert struct.unpack("<f", blob[-4:])[0] == np.float32(1e-12)
+    assert c.deserializePlugin("ln", blob).serialize() == blob
+
+    with pytest.raises(lib.FwdmiError, match="int8"):
+        c.createPlugin("ln", ln_fields(8, lib.I8, rng))
+    with pytest.raises(lib.FwdmiError, match="Invalid type ID"):
+        c.createPlugin("ln", ln_fields(8, 7, rng))
+    with pytest.raises(lib.FwdmiError, match="ld=9"):
+        c.createPlugin("ln", [F("ld", 9)] + ln_fields(8, lib.F32, rng)[1:])
+
+
+def emb_fields(rng, ld=16, vocab=40, pos=12, fp16=0):
+    # names and order of trt_bert_creator.h:130-141
+    r = lambda *s: rng.standard_normal(s).astype(np.float32)
+    return [F("bert_embeddings_layernorm_beta", r(ld)), F("bert_embeddings_layernorm_gamma", r(ld)),
+            F("bert_embeddings_word_embeddings", r(vocab, ld)), F("bert_embeddings_token_type_embeddings", r(2, ld)),
+            F("bert_embeddings_position_embeddings", r(pos, ld)), F("output_fp16", fp16), F("mha_type_id", fp16)]
+
+
+def test_emb_layer_norm_plugin_host_contract():
+    rng = np.random.default_rng(3)
+    c = REG.getPluginCreator("CustomEmbLayerNormPluginDynamic", "1")
+    fields = emb_fields(rng, fp16=1)
+    p = c.createPlugin("embeddings", fields)
+    assert p.getNbOutputs() == 2
+    ins = [(12, 4)] * 3                                                       # [S, B]
+    assert p.getOutputDimensions(0, ins) == [12, 4, 16, 1, 1]                 # consumed as [S,B,H,1,1]
+    assert p.getOutputDimensions(1, ins) == [4, 1]                            # one mask index per batch row
+    with pytest.raises(lib.FwdmiError):
+        p.getOutputDimensions(0, [(12, 4), (12, 4), (12, 5)])
+    io = [((12, 4), lib.I32)] * 3 + [((12, 4, 16, 1, 1), lib.F16), ((4, 1), lib.I32)]
+    assert all(p.supportsFormatCombination(i, io, 3, 2) for i in range(5))
+    assert not p.supportsFormatCombination(3, io[:3] + [((12, 4, 16, 1, 1), lib.F32), io[4]], 3, 2)
+    assert p.getOutputDataType(0, [lib.I32] * 3) == lib.F16 and p.getOutputDataType(1, [lib.I32] * 3) == lib.I32
+    blob = p.serialize()
+    assert struct.unpack("<6if", blob[:28]) == (lib.F16, lib.F16, 16, 40, 12, 2, 0.0)
+    assert blob[28:28 + 64] == fields[0].array.tobytes()
+    assert blob[28 + 128:28 + 128 + 40 * 16 * 2] == fields[2].array.astype(np.float16).tobytes()
+    assert len(blob) == p.getSerializationSize() == 28 + 128 + (40 + 12 + 2) * 16 * 2
+    assert c.deserializePlugin("e", blob).serialize() == blob and p.clone().serialize() == blob
+    with pytest.raises(lib.FwdmiError):
+        c.deserializePlugin("e", blob[:-1])
+    with pytest.raises(lib.FwdmiError, match="inconsistent sizes"):
+        c.createPlugin("e", fields[:2] + [F("bert_embeddings_word_embeddings", np.zeros(17, np.float32))] + fields[3:])

@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Benchmark of the embedding-side hot path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config4] [--no-cpu] [--no-extra]
+
+A step is one pass of the DLRM-style sparse stage (BASELINE config 4): 26 sum-mode tables, fp16
+rows of dim 128, 65536 bags per table with truncated-Zipf lengths, Zipf ids, fp16 output
+concatenated to [65536, 3328], issued as ONE fused launch.  Inputs are resident in HBM before the
+timed region.  Prints one JSON line: bags/s over the whole job, the HBM-roofline position of the
+kernel from HIP-event timing of the same launches, and a CPU baseline (the C oracle and libtorch
+CPU) timed on this box's host cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBS = 8000.0
+ROOT = os.path.dirname(os.path.abspath(__file__))
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="config4", choices=["config4"])
+    ap.add_argument("--tables", type=int, default=26, help="debug only: fewer tables (not the named config)")
+    ap.add_argument("--bags", type=int, default=65536, help="debug only: smaller batch (not the named config)")
+    ap.add_argument("--per-table", action="store_true", help="26 launches instead of the fused one")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--no-extra", action="store_true", help="skip the config 2/3/5 side measurements")
+    ap.add_argument("--cpu-bags", type=int, default=4096, help="bags per table in the CPU baseline sample")
+    return ap.parse_args()
+
+
+def device_tables(wl, torch):
+    """fp16 rows ~U(-0.05, 0.05) generated in HBM (seeded per table)."""
+    tabs = []
+    for t, rows in enumerate(wl.rows):
+        g = torch.Generator(device="cuda").manual_seed(wl.table_seeds[t])
+        x = torch.rand((rows, wl.dim), generator=g, device="cuda", dtype=torch.float32)
+        tabs.append(((x - 0.5) * 0.1).to(torch.float16))
+        del x
+    return tabs
+
+
+def time_events(torch, fn, steps, warmup):
+    """Wall-clock over `steps` back-to-back calls plus per-call HIP-event durations (ms)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = np.array([a.elapsed_time(b) for a, b in evs])
+    return wall, per
+
+
+def cpu_baseline(wl, tabs_dev, n_cpu_bags, torch):
+    """The C oracle ("port") and libtorch CPU on the first `n_cpu_bags` bags of every table."""
+    from oracle import oracle          # checker, used here only as the timed CPU baseline
+    oracle.build()
+    cores = min(16, os.cpu_count() or 1)
+    oracle.set_threads(cores)
+    nb = min(n_cpu_bags, wl.n_bags)
+    host_tabs, idxs, offs = [], [], []
+    for t in range(len(wl.rows)):
+        end = int(wl.offsets[t][nb]) if nb < wl.n_bags else wl.indices[t].size
+        host_tabs.append(tabs_dev[t].cpu().numpy())
+        idxs.append(np.ascontiguousarray(wl.indices[t][:end]))
+        offs.append(np.ascontiguousarray(wl.offsets[t][:nb]))
+    total_bags = nb * len(wl.rows)
+    out = np.zeros((nb, len(wl.rows) * wl.dim), np.float16)
+
+    def run_oracle():
+        for t in range(len(wl.rows)):
+            oracle.embedding_bag(host_tabs[t], idxs[t], offs[t], oracle.OP_SUM, out=out, out_col=t * wl.dim)
+
+    def timed(fn, budget_s=8.0, min_reps=2):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if reps >= min_reps and dt > budget_s or reps >= 20:
+                return dt / reps
+
+    res = {"unit": "bags/s", "kind": "port", "cores": cores,
+           "sample": "all %d tables x first %d of %d bags, same ids/offsets, C oracle with OpenMP" %
+                     (len(wl.rows), nb, wl.n_bags)}
+    res["value"] = total_bags / timed(run_oracle)
+    # libtorch CPU, the ground truth the reference's own tests use
+    tt = [torch.from_numpy(a) for a in host_tabs]
+    ti = [torch.from_numpy(a) for a in idxs]
+    to = [torch.from_numpy(a) for a in offs]
+
+    def run_torch():
+        return torch.cat([torch.nn.functional.embedding_bag(ti[t], tt[t], to[t], mode="sum")
+                          for t in range(len(tt))], dim=1)
+
+    lt = {}
+    for n in (cores, 1):
+        torch.set_num_threads(n)
+        lt["threads_%d" % n] = total_bags / timed(run_torch, budget_s=5.0)
+    torch.set_num_threads(cores)
+    res["libtorch_cpu_bags_per_s"] = lt
+    try:
+        with open("/proc/cpuinfo") as f:
+            res["cpu_model"] = next(l.split(":", 1)[1].strip() for l in f if l.startswith("model name"))
+    except Exception:
+        pass
+    # the sample doubles as a spot check of the GPU result
+    return res, out, nb
+
+
+def extra_measurements(torch, ops, workloads, steps):
+    """Tokens/s of the BERT configs and bags/s of config 2 (side measurements, HIP-event timed)."""
+    ex = {}
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    f32 = lambda a: dev(np.asarray(a, np.float32))
+    for name, wl in (("config3_emb_layer_norm", workloads.config3()), ("config5_emb_layer_norm", workloads.config5())):
+        a = [dev(wl.input_ids), dev(wl.segment_ids), dev(wl.input_mask), dev(wl.word), dev(wl.pos), dev(wl.tok),
+             f32(wl.gamma), f32(wl.beta)]
+        out = torch.empty((wl.input_ids.shape[0], wl.input_ids.shape[1], wl.word.shape[1]), dtype=torch.float16,
+                          device="cuda")
+        midx = torch.empty((wl.input_ids.shape[1],), dtype=torch.int32, device="cuda")
+        fn = lambda: ops.emb_layer_norm(*a, eps=wl.eps, out=out, mask_idx=midx)
+        _, per = time_events(torch, fn, steps, 5)
+        ms = float(np.median(per))
+        ex[name] = {"tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
+                    "algorithmic_GBs": wl.emb_algorithmic_bytes() / (ms * 1e-3) / 1e9}
+        if wl.skip is not None:
+            x, sk = out, dev(wl.skip)
+            g, b, bi = f32(wl.skip_gamma), f32(wl.skip_beta), f32(wl.skip_bias)
+            o2 = torch.empty_like(x)
+            fn2 = lambda: ops.skip_layer_norm(x, g, b, skip=sk, bias=bi, eps=wl.eps, out=o2)
+            _, per = time_events(torch, fn2, steps, 5)
+            ms = float(np.median(per))
+            ex["config5_skip_layer_norm"] = {"tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
+                                             "algorithmic_GBs": wl.skip_algorithmic_bytes() / (ms * 1e-3) / 1e9}
+    for tdt, tname in ((np.float32, "fp32"), (np.float16, "fp16")):
+        wl = workloads.config2(table_dtype=tdt)
+        tb, ix, of = dev(wl.table), dev(wl.indices), dev(wl.offsets)
+        out = torch.empty((wl.n_bags, 128), dtype=tb.dtype, device="cuda")
+        fn = lambda: ops.embedding_bag(tb, ix, of, "sum", out=out)
+        _, per = time_events(torch, fn, steps, 5)
+        ms = float(np.median(per))
+        ex["config2_sum_%s_int32" % tname] = {"bags_per_s": wl.n_bags / (ms * 1e-3), "ms": ms,
+                                              "algorithmic_GBs": wl.algorithmic_bytes() / (ms * 1e-3) / 1e9}
+    return ex
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (got --gpus %d)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from forward_amd import ops, workloads
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+
+    t0 = time.time()
+    wl = workloads.config4(n_tables=args.tables, n_bags=args.bags)
+    log("ids/offsets generated in %.1fs: %d tables, %d bags each, %d ids, rows %s" %
+        (time.time() - t0, len(wl.rows), wl.n_bags, wl.n_indices(), wl.rows))
+    tabs = device_tables(wl, torch)
+    idx = [torch.from_numpy(i).cuda() for i in wl.indices]
+    off = [torch.from_numpy(o).cuda() for o in wl.offsets]
+    batch = ops.MultiTableBatch(tabs, idx, off)
+    out = torch.zeros((wl.n_bags, batch.width), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    log("tables resident: %.2f GB, setup %.1fs" % (sum(t.numel() * 2 for t in tabs) / 1e9, time.time() - t0))
+
+    if args.per_table:
+        def step():
+            for t in range(batch.n_tables):
+                ops.embedding_bag(tabs[t], idx[t], off[t], "sum", out=out, out_col=t * wl.dim)
+        launches_per_step = batch.n_tables
+    else:
+        def step():
+            batch.forward(out=out)
+        launches_per_step = 1
+
+    wall, per = time_events(torch, step, args.steps, args.warmup)
+    ms_per_step = wall / args.steps * 1e3
+    total_bags = wl.n_bags * len(wl.rows)
+    alg_bytes = wl.algorithmic_bytes(table_itemsize=2, out_itemsize=2, index_itemsize=4)
+    ev_ms = float(np.mean(per))
+    achieved = alg_bytes / (ev_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "EmbeddingBag bags/sec + achieved HBM GB/s (% peak), 26-table fp16 batch 64K",
+        "value": total_bags / (ms_per_step * 1e-3), "unit": "bags/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 rows, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "config4: DLRM sparse stage, %d tables x %d bags, dim %d fp16, int32 ids, "
+                               "Zipf(1.1) ids and bag lengths (mean %.2f), fp16 output [%d, %d]%s"
+                               % (len(wl.rows), wl.n_bags, wl.dim, wl.n_indices() / total_bags, wl.n_bags,
+                                  batch.width, "" if (args.tables == 26 and args.bags == 65536) else " (REDUCED, debug)"),
+                   "launch": "per-table" if args.per_table else "fused multi-table",
+                   "total_ids": wl.n_indices(), "table_bytes": int(sum(t.numel() * 2 for t in tabs))},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": alg_bytes / launches_per_step,
+                     "kernel_ms_avg": ev_ms / launches_per_step, "kernel_ms_p10": float(np.percentile(per, 10)),
+                     "kernel_ms_p90": float(np.percentile(per, 90)), "launches_per_step": launches_per_step},
+        "samples_per_s": wl.n_bags / (ms_per_step * 1e-3),
+    }
+    prof = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(prof) and not args.per_table and args.tables == 26 and args.bags == 65536:
+        with open(prof) as f:
+            result["roofline"]["traffic"] = json.load(f).get("bag_reduce_config4_bytes_per_launch")
+
+    if not args.no_cpu:
+        t1 = time.time()
+        cpu, cpu_out, nb = cpu_baseline(wl, tabs, args.cpu_bags, torch)
+        gpu_out = out[:nb].cpu().numpy()
+        cpu["gpu_matches_oracle_on_sample"] = bool(np.array_equal(gpu_out.view(np.uint16), cpu_out.view(np.uint16)))
+        result["cpu_baseline"] = cpu
+        log("cpu baseline leg %.1fs" % (time.time() - t1))
+    if not args.no_extra:
+        del tabs, batch
+        result["extra"] = extra_measurements(torch, ops, workloads, max(10, args.steps))
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -7,6 +7,13 @@ so a fresh checkout works, and a failure to build or load raises ``ImportError``
 import ctypes as C
 import os
 
+# PyTorch-ROCm wheels bundle their own HIP runtime whose SONAME (libamdhip64.so.7) equals the
+# system one libfwdmi.so is linked against.  Importing torch first makes the dynamic loader
+# resolve libfwdmi.so's dependency to the runtime torch already loaded; the other order puts
+# two HIP runtimes into one process, and device pointers / streams from one are garbage to
+# the other.
+import torch  # noqa: F401  (must precede the CDLL below)
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfwdmi.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "fwdmi.h")

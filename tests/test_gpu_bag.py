@@ -1,0 +1,249 @@
+"""GPU parity of the bag-reduction kernels against the CPU oracle, through the C ABI
+(kernel launchers and plugin objects).  Integer work (ids, argmax, empty bags) is bit-exact;
+because rows are summed in bag order with the oracle's operations, fp32 and fp16 values are
+bit-exact too, which is stricter than the stated tolerance (also asserted)."""
+import numpy as np
+import pytest
+import torch
+
+from forward_amd import lib, ops, plugin, workloads
+from forward_amd.plugin import PluginFieldData as F
+from gpu_util import assert_bits_equal, assert_close, dev, host
+
+pytestmark = pytest.mark.gpu
+
+OPS = {"sum": 0, "mean": 1, "max": 2, "square_sum": 3}
+
+
+def run_bag(wl_table, idx, off, mode, psw=None, **kw):
+    return ops.embedding_bag(dev(wl_table), dev(idx), dev(off), mode, per_sample_weights=dev(psw), **kw)
+
+
+def test_config1_exact(oracle):
+    wl = workloads.config1()
+    got = host(run_bag(wl.table, wl.indices, wl.offsets, "sum"))
+    want, _, _ = oracle.embedding_bag(wl.table, wl.indices, wl.offsets, oracle.OP_SUM)
+    assert_bits_equal(got, want, "config 1")
+    ref = torch.nn.functional.embedding_bag(torch.from_numpy(wl.indices), torch.from_numpy(wl.table),
+                                            torch.from_numpy(wl.offsets), mode="sum").numpy()
+    assert_close(got, ref, np.float32)
+
+
+@pytest.mark.parametrize("tdt", [np.float32, np.float16])
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+@pytest.mark.parametrize("mode", ["sum", "mean", "max", "wsum"])
+def test_config2_scaled(oracle, tdt, idt, mode):
+    weighted = mode == "wsum"
+    m = "sum" if weighted else mode
+    wl = workloads.config2(variant=1, table_dtype=tdt, index_dtype=idt, mode=m, weighted=weighted, rows=60000)
+    assert (wl.lengths == 0).sum() > 10 and wl.lengths.max() > 30
+    res = run_bag(wl.table, wl.indices, wl.offsets, m, wl.per_sample_weights, want_max_indices=(m == "max"))
+    want, warg, oob = oracle.embedding_bag(wl.table, wl.indices, wl.offsets, OPS[m],
+                                           per_sample_weights=wl.per_sample_weights, want_max_indices=(m == "max"))
+    assert oob == 0
+    got = host(res[0] if m == "max" else res)
+    assert got.dtype == tdt
+    assert_close(got, want, tdt, scale=0.05)
+    assert_bits_equal(got, want, "values")
+    empty = wl.lengths == 0
+    assert not got[empty].any()
+    if m == "max":
+        arg = host(res[1])
+        assert arg.dtype == idt
+        np.testing.assert_array_equal(arg, warg)
+
+
+def test_config2_full_size_sum_fp16(oracle):
+    wl = workloads.config2(variant=0, table_dtype=np.float16, index_dtype=np.int32)
+    assert wl.table.shape == (1_000_000, 128) and wl.n_bags == 4096
+    got = host(run_bag(wl.table, wl.indices, wl.offsets, "sum"))
+    want, _, _ = oracle.embedding_bag(wl.table, wl.indices, wl.offsets, oracle.OP_SUM)
+    assert_close(got, want, np.float16)
+    assert_bits_equal(got, want, "config 2 fp16")
+
+
+@pytest.mark.parametrize("dim,tdt", [(1, np.float32), (2, np.float32), (4, np.float32), (10, np.float16),
+                                     (64, np.float32), (100, np.float16), (200, np.float32), (1024, np.float16),
+                                     (1100, np.float32), (2048, np.float32)])
+def test_row_widths(oracle, dim, tdt):
+    rng = np.random.Generator(np.random.PCG64(dim))
+    table = rng.standard_normal((300, dim)).astype(tdt)
+    lengths = rng.integers(0, 12, size=97)
+    idx = rng.integers(0, 300, size=int(lengths.sum())).astype(np.int32)
+    off = workloads.offsets_from_lengths(lengths, np.int32)
+    for mode in ("sum", "max"):
+        got = host(run_bag(table, idx, off, mode))
+        want, _, _ = oracle.embedding_bag(table, idx, off, OPS[mode])
+        assert_bits_equal(got, want, "dim %d %s" % (dim, mode))
+
+
+def test_long_bags_exceed_lds_window(oracle):
+    rng = np.random.Generator(np.random.PCG64(77))
+    table = rng.standard_normal((4000, 128)).astype(np.float16)
+    lengths = np.array([0, 5000, 1, 2047, 2049, 0, 9000, 3], np.int64)
+    idx = rng.integers(0, 4000, size=int(lengths.sum())).astype(np.int64)
+    off = workloads.offsets_from_lengths(lengths, np.int64)
+    psw = rng.random(idx.size).astype(np.float16)
+    for mode, w in (("sum", None), ("mean", None), ("max", None), ("sum", psw)):
+        got = host(run_bag(table, idx, off, mode, w))
+        want, _, _ = oracle.embedding_bag(table, idx, off, OPS[mode], per_sample_weights=w)
+        assert_bits_equal(got, want, "long bags %s" % mode)
+
+
+def test_out_of_range_ids_are_skipped_and_flagged(oracle):
+    table = (np.arange(40, dtype=np.float32).reshape(10, 4) + 1)
+    idx = np.array([100, 103, 99, 110, 109, -1, 2**31 - 1, 105], np.int32)      # shard holds ids 100..109
+    off = np.array([0, 3, 3], np.int32)
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    got = host(run_bag(table, idx, off, "sum", data_offset=100, oob_flag=flag))
+    want, _, oob = oracle.embedding_bag(table, idx, off, oracle.OP_SUM, data_offset=100)
+    assert oob == 4
+    assert_bits_equal(got, want, "filtered")
+    assert int(flag.item()) == 1
+    flag.zero_()
+    run_bag(table, np.array([100, 109], np.int32), np.array([0], np.int32), "sum", data_offset=100, oob_flag=flag)
+    assert int(flag.item()) == 0
+    # 64-bit ids far outside the table
+    idx64 = np.array([5, 2**40, -2**40, 9], np.int64)
+    got = host(run_bag(table, idx64, np.array([0], np.int64), "sum"))
+    np.testing.assert_array_equal(got[0], table[5] + table[9])
+
+
+def test_include_last_offset_and_empty_batches(oracle):
+    wl = workloads.config2(variant=4, rows=3000, n_bags=50)
+    off_last = np.append(wl.offsets, wl.indices.size).astype(np.int32)
+    a = host(run_bag(wl.table, wl.indices, wl.offsets, "sum"))
+    b = host(run_bag(wl.table, wl.indices, off_last, "sum", include_last_offset=True))
+    assert_bits_equal(a, b, "include_last_offset")
+    # all bags empty / no ids at all
+    z = host(run_bag(wl.table, np.zeros(0, np.int32), np.zeros(7, np.int32), "max"))
+    assert z.shape == (7, 128) and not z.any()
+    # zero bags: nothing launched, nothing written
+    e = ops.embedding_bag(dev(wl.table), dev(np.zeros(0, np.int32)), dev(np.zeros(0, np.int32)), "sum")
+    assert e.shape == (0, 128)
+
+
+def test_fixed_length_square_sum_and_gather(oracle):
+    rng = np.random.Generator(np.random.PCG64(21))
+    table = rng.standard_normal((50, 6)).astype(np.float32)
+    idx = rng.integers(0, 50, size=(10, 5)).astype(np.int32)                   # test_tf_nodes.h:199-211 shape
+    for mode in ("sum", "square_sum", "mean", "max"):
+        got = host(ops.embedding_bag_fixed(dev(table), dev(idx), mode))
+        want, _, _ = oracle.embedding_bag(table, idx, None, OPS[mode])
+        assert_bits_equal(got, want, "fixed %s" % mode)
+    g = host(ops.gather(dev(table), dev(idx)))
+    want, _ = oracle.gather(table, idx)
+    assert_bits_equal(g, want, "gather")
+    big = rng.standard_normal((1000, 128)).astype(np.float16)
+    ids = rng.integers(-3, 1003, size=(1, 1000)).astype(np.int64)
+    g = host(ops.gather(dev(big), dev(ids), out_dtype=torch.float32))
+    want, oob = oracle.gather(big, ids, out_dtype=np.float32)
+    assert oob > 0
+    assert_bits_equal(g, want, "gather fp16->fp32")
+
+
+def test_multi_table_concatenated(oracle):
+    wl = workloads.config4(variant=2, n_tables=5, n_bags=3000, max_rows=30000)
+    tabs = [wl.host_table(t) for t in range(5)]
+    want = np.zeros((3000, 5 * 128), np.float16)
+    for t in range(5):
+        oracle.embedding_bag(tabs[t], wl.indices[t], wl.offsets[t], oracle.OP_SUM, out=want, out_col=128 * t)
+    batch = ops.MultiTableBatch([dev(t) for t in tabs], [dev(i) for i in wl.indices], [dev(o) for o in wl.offsets])
+    got = host(batch.forward())
+    assert_bits_equal(got, want, "fused multi-table")
+    # the same through 5 single-table launches writing column blocks
+    out = torch.zeros((3000, 640), dtype=torch.float16, device="cuda")
+    for t in range(5):
+        ops.embedding_bag(batch.tables[t], batch.indices[t], batch.offsets[t], "sum", out=out, out_col=128 * t)
+    assert_bits_equal(host(out), want, "per-table launches")
+    got32 = host(batch.forward(out_dtype=torch.float32))
+    np.testing.assert_allclose(got32, want.astype(np.float32), atol=1e-2, rtol=5e-3)
+
+
+# ---- through the plugin objects ------------------------------------------------------------------
+REG = plugin.getPluginRegistry()
+
+
+def bag_fields(table, op=0, offset=0):
+    count, dim = table.shape
+    return [F("dim", dim), F("count", count), F("offset", offset), F("op", op), F("data", table)]
+
+
+def test_plugin_reference_known_answers(kats):
+    k = kats["embedding_bag_module"]
+    w = np.array(k["table"], np.float32)
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    p = c.createPlugin("embedding_bag", bag_fields(w))
+    # the reference engine feeds int64 ids as int32 (torch_engine.cpp:134-149)
+    out = host(p(dev(np.array(k["indices"], np.int32)), dev(np.array(k["offsets"], np.int32))))
+    want = np.zeros((5, 4))
+    want[4] = (w[0].astype(np.float64) + 2 * w[1].astype(np.float64) + w[3] + w[4])
+    np.testing.assert_allclose(out, want, atol=1e-3)           # the reference test's threshold
+    np.testing.assert_allclose(out, want, rtol=1e-6, atol=1e-7)
+    assert not out[:4].any()
+
+    d = kats["dlrm"]
+    expect = [[[0.48071694, 0.18480009], [0.41585842, -0.29087239]],
+              [[-0.18103497, 0.26449448], [-0.25194445, -0.24395032]],
+              [[-0.44896644, -0.45899662], [-0.44896644, -0.45899662]]]
+    for t in range(3):
+        tab = np.array(d["tables"][t], np.float32)
+        q = c.createPlugin("emb_%d" % t, bag_fields(tab))
+        off = np.array(d["offsets"][t], np.int32).reshape(1, 2)          # DLRM passes a [1, B] slice
+        out = host(q(dev(np.array(d["indices"][t], np.int32)), dev(off)))
+        np.testing.assert_allclose(out, expect[t], atol=1e-4)           # test_torch_dlrm.h:56
+        np.testing.assert_allclose(out, expect[t], rtol=1e-6, atol=1e-7)
+
+
+def test_plugin_serialize_load_run_matches(oracle):
+    """Build -> save -> load -> run, as the reference's test harness does (unit_test_torch_helper.h:79-138)."""
+    wl = workloads.config1()
+    idx, off = wl.indices.astype(np.int32), wl.offsets.astype(np.int32)
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    p = c.createPlugin("embedding_bag", bag_fields(wl.table))
+    direct = host(p(dev(idx), dev(off)))
+    loaded = c.deserializePlugin("embedding_bag", p.serialize())
+    again = host(loaded(dev(idx), dev(off)))
+    clone = loaded.clone()
+    third = host(clone(dev(idx), dev(off)))
+    want, _, _ = oracle.embedding_bag(wl.table, idx, off, oracle.OP_SUM)
+    for got in (direct, again, third):
+        assert_bits_equal(got, want, "plugin")
+    loaded.destroy()                     # the clone keeps the shared device table alive
+    assert_bits_equal(host(clone(dev(idx), dev(off))), want, "clone after destroy")
+    # wrong id type is refused with -1, as in the reference
+    rc = p.enqueue_raw([((idx.size,), lib.I64), ((64,), lib.I64)], [((64, 64), lib.F32)], [0, 0], [0])
+    assert rc == lib.ERR_UNSUPPORTED
+
+
+def test_plugin_modes_fixed_gather_and_extended(oracle):
+    rng = np.random.Generator(np.random.PCG64(31))
+    table = rng.standard_normal((50, 8)).astype(np.float32)
+    idx2d = rng.integers(0, 50, size=(10, 5)).astype(np.int32)
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    for op in (0, 3):                                               # SUM and SQUARE_SUM: what the TF front end emits
+        got = host(c.createPlugin("fm", bag_fields(table, op=op))(dev(idx2d)))
+        want, _, _ = oracle.embedding_bag(table, idx2d, None, op)
+        assert_bits_equal(got, want, "fixed op %d" % op)
+    g = host(c.createPlugin("gather", bag_fields(table, op=999))(dev(idx2d)))
+    assert g.shape == (10, 5, 8)
+    assert_bits_equal(g, table[idx2d], "plugin gather")
+    # torch mode ints 1 / 2 mean MEAN / MAX
+    wl = workloads.config2(variant=5, rows=2000, n_bags=200)
+    for op in (1, 2):
+        got = host(c.createPlugin("bag", bag_fields(wl.table, op=op))(dev(wl.indices), dev(wl.offsets)))
+        want, _, _ = oracle.embedding_bag(wl.table, wl.indices, wl.offsets, op)
+        assert_bits_equal(got, want, "plugin op %d" % op)
+    # extended contract: fp16 table, int64 ids, fp16 output, per-sample weights, trailing offset
+    c2 = REG.getPluginCreator("EmbeddingBag_TRT", "002")
+    t16 = wl.table.astype(np.float16)
+    psw = rng.random(wl.indices.size).astype(np.float16)
+    p = c2.createPlugin("bag", bag_fields(t16) + [F("index_type", lib.I64), F("output_fp16", 1),
+                                                  F("include_last_offset", 1), F("per_sample_weights", 1)])
+    i64 = wl.indices.astype(np.int64)
+    o64 = np.append(wl.offsets, wl.indices.size).astype(np.int64)
+    got = host(p(dev(i64), dev(o64), dev(psw)))
+    want, _, _ = oracle.embedding_bag(t16, i64, o64, 0, per_sample_weights=psw, include_last_offset=True)
+    assert got.dtype == np.float16 and got.shape == (200, 128)
+    assert_bits_equal(got, want, "extended plugin")
+    assert not p.takeOobFlag()

@@ -1,0 +1,169 @@
+"""GPU parity of the LayerNorm-family kernels against the CPU oracle (float64 closed form),
+through the C ABI launchers and the plugin objects.  Tolerances: fp32 rel 1e-5 (abs 1e-5 floor,
+outputs are O(1)); fp16 abs 1e-2 / rel 5e-3; the mask index is bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from forward_amd import lib, ops, plugin, workloads
+from forward_amd.plugin import PluginFieldData as F
+from gpu_util import assert_close, dev, host
+
+pytestmark = pytest.mark.gpu
+REG = plugin.getPluginRegistry()
+
+
+def f32(a):
+    return dev(np.asarray(a, np.float32))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_config3_emb_layer_norm(oracle, dtype):
+    wl = workloads.config3(dtype=dtype)
+    assert wl.input_ids.shape == (128, 32) and wl.word.shape == (30522, 768)
+    out, midx = ops.emb_layer_norm(dev(wl.input_ids), dev(wl.segment_ids), dev(wl.input_mask), dev(wl.word),
+                                   dev(wl.pos), dev(wl.tok), f32(wl.gamma), f32(wl.beta), eps=wl.eps)
+    want, wmidx, oob = oracle.emb_layer_norm(wl.input_ids, wl.segment_ids, wl.input_mask, wl.word, wl.pos, wl.tok,
+                                             wl.gamma, wl.beta, eps=wl.eps)
+    assert oob == 0
+    assert_close(host(out), want, dtype)
+    np.testing.assert_array_equal(host(midx), wmidx)
+    np.testing.assert_array_equal(host(midx), wl.valid_len)
+    if dtype == np.float16:
+        # next to the oracle: libtorch CPU's own fp16 path (embedding x3, add, layer_norm, rounding per op)
+        S = wl.input_ids.shape[0]
+        tw, tp, tt = (torch.from_numpy(a) for a in (wl.word, wl.pos, wl.tok))
+        e = (torch.nn.functional.embedding(torch.from_numpy(wl.input_ids).long(), tw) + tp[:S].unsqueeze(1)
+             + torch.nn.functional.embedding(torch.from_numpy(wl.segment_ids).long(), tt))
+        ref = torch.nn.functional.layer_norm(e.float(), (768,), torch.from_numpy(wl.gamma).float(),
+                                             torch.from_numpy(wl.beta).float(), wl.eps)
+        assert_close(host(out), ref.numpy(), np.float16)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_config5_emb_then_skip_layer_norm(oracle, dtype):
+    wl = workloads.config5(dtype=dtype)
+    assert wl.input_ids.shape == (512, 16) and wl.skip.shape == (512, 16, 1024)
+    emb, midx = ops.emb_layer_norm(dev(wl.input_ids), dev(wl.segment_ids), dev(wl.input_mask), dev(wl.word),
+                                   dev(wl.pos), dev(wl.tok), f32(wl.gamma), f32(wl.beta), eps=wl.eps)
+    out = ops.skip_layer_norm(emb, f32(wl.skip_gamma), f32(wl.skip_beta), skip=dev(wl.skip), bias=f32(wl.skip_bias),
+                              eps=wl.eps)
+    wemb, wmidx, _ = oracle.emb_layer_norm(wl.input_ids, wl.segment_ids, wl.input_mask, wl.word, wl.pos, wl.tok,
+                                           wl.gamma, wl.beta, eps=wl.eps)
+    assert_close(host(emb), wemb, dtype)
+    np.testing.assert_array_equal(host(midx), wmidx)
+    # second stage checked on the GPU's own first-stage output, so errors do not compound
+    want = oracle.skip_layer_norm(host(emb), wl.skip_gamma, wl.skip_beta, skip=wl.skip, bias=wl.skip_bias, eps=wl.eps)
+    assert_close(host(out), want, dtype)
+
+
+@pytest.mark.parametrize("ld,dtype", [(1, np.float32), (7, np.float32), (10, np.float32), (32, np.float16),
+                                      (48, np.float32), (100, np.float16), (256, np.float32), (768, np.float32),
+                                      (1000, np.float16), (1024, np.float16), (4096, np.float16),
+                                      (2048, np.float32), (5000, np.float32), (8192, np.float16)])
+def test_layer_norm_row_lengths(oracle, ld, dtype):
+    rng = np.random.Generator(np.random.PCG64(ld))
+    x = (rng.standard_normal((37, ld)) * 2 + 0.5).astype(dtype)
+    sk = rng.standard_normal((37, ld)).astype(dtype)
+    g = (1 + 0.1 * rng.standard_normal(ld)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(ld)).astype(np.float32)
+    bi = (0.1 * rng.standard_normal(ld)).astype(np.float32)
+    eps = 1e-5
+    got = host(ops.layer_norm(dev(x), dev(g), dev(b), eps=eps))
+    assert_close(got, oracle.layer_norm(x, g, b, eps=eps), dtype)
+    got = host(ops.layer_norm(dev(x), dev(g), dev(b), bias=dev(bi), eps=eps))
+    assert_close(got, oracle.layer_norm(x, g, b, bias=bi, eps=eps), dtype)
+    got = host(ops.skip_layer_norm(dev(x), dev(g), dev(b), skip=dev(sk), bias=dev(bi), eps=eps))
+    assert_close(got, oracle.skip_layer_norm(x, g, b, skip=sk, bias=bi, eps=eps), dtype)
+
+
+def test_layer_norm_large_mean_is_stable(oracle):
+    """|mean| >> std: the E[x^2]-mean^2 form of the reference loses all digits here; Welford does not."""
+    rng = np.random.Generator(np.random.PCG64(9))
+    x = (1000.0 + 0.1 * rng.standard_normal((64, 1024))).astype(np.float32)
+    g, b = np.ones(1024, np.float32), np.zeros(1024, np.float32)
+    got = host(ops.layer_norm(dev(x), dev(g), dev(b), eps=0.0))
+    want = oracle.layer_norm(x, g, b, eps=0.0)
+    np.testing.assert_allclose(got, want, rtol=1e-3, atol=1e-3)
+    assert np.isfinite(got).all()
+
+
+def test_many_rows_loop_path(oracle):
+    rng = np.random.Generator(np.random.PCG64(10))
+    x = rng.standard_normal((20000, 64)).astype(np.float16)     # more rows than wavefronts in the grid
+    g, b = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32), (0.1 * rng.standard_normal(64)).astype(np.float32)
+    got = host(ops.layer_norm(dev(x), dev(g), dev(b), eps=1e-5))
+    assert_close(got, oracle.layer_norm(x, g, b, eps=1e-5), np.float16)
+
+
+def test_emb_layer_norm_mask_and_out_of_table_ids(oracle):
+    wl = workloads.config3(variant=7, dtype=np.float32, batch=5, seq=70)
+    ids, seg, msk = wl.input_ids.copy(), wl.segment_ids.copy(), wl.input_mask.copy()
+    msk[3, 1] = 0                      # a hole: mask index is the first zero, not the count of ones
+    msk[:, 4] = 1                      # no zero at all -> S
+    ids[2, 0] = 40000                  # outside the word table: contributes a zero row, raises the flag
+    seg[6, 3] = 9
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    out, midx = ops.emb_layer_norm(dev(ids), dev(seg), dev(msk), dev(wl.word), dev(wl.pos), dev(wl.tok),
+                                   f32(wl.gamma), f32(wl.beta), eps=wl.eps, oob_flag=flag)
+    want, wmidx, oob = oracle.emb_layer_norm(ids, seg, msk, wl.word, wl.pos, wl.tok, wl.gamma, wl.beta, eps=wl.eps)
+    assert oob == 2 and int(flag.item()) == 1
+    assert_close(host(out), want, np.float32)
+    np.testing.assert_array_equal(host(midx), wmidx)
+    assert wmidx[1] == 3 and wmidx[4] == 70
+
+
+# ---- through the plugin objects ------------------------------------------------------------------
+def test_plugin_layer_norm_with_weights_reference_shape(oracle, kats):
+    """test_torch_nodes.h:293-299: input [20,5,10], LayerNorm(10) with the stored weights, threshold 1e-3."""
+    k = kats["layer_norm_with_weights"]
+    a, b = np.array(k["data0"], np.float32), np.array(k["data1"], np.float32)
+    gamma, beta = (a, b) if a.sum() > b.sum() else (b, a)
+    c = REG.getPluginCreator("ForwardLayerNormPluginDynamic", "1")
+    # fields as trt_normalization_creator.h:147-157 sends them (no eps reaches the plugin)
+    p = c.createPlugin("skip_layer_norm", [F("ld", 10), F("beta", beta), F("gamma", gamma), F("type_id", lib.F32),
+                                           F("has_skip", 0), F("batch_size", 20)])
+    x = np.random.Generator(np.random.PCG64(12)).standard_normal(k["input_shape"]).astype(np.float32)
+    out = host(p(dev(x)))
+    ref = torch.nn.functional.layer_norm(torch.from_numpy(x), (10,), torch.from_numpy(gamma), torch.from_numpy(beta),
+                                         k["eps"]).numpy()
+    np.testing.assert_allclose(out, ref, atol=1e-3)
+    assert_close(out, oracle.layer_norm(x, gamma, beta, eps=0.0), np.float32)
+    again = host(c.deserializePlugin("ln", p.serialize())(dev(x)))
+    np.testing.assert_array_equal(out, again)
+
+
+def test_plugins_config5_chain(oracle):
+    wl = workloads.config5(variant=1, batch=4, seq=64)
+    up = lambda a: a.astype(np.float32)
+    ce = REG.getPluginCreator("CustomEmbLayerNormPluginDynamic", "1")
+    emb = ce.createPlugin("embeddings", [
+        F("bert_embeddings_layernorm_beta", up(wl.beta)), F("bert_embeddings_layernorm_gamma", up(wl.gamma)),
+        F("bert_embeddings_word_embeddings", up(wl.word)), F("bert_embeddings_token_type_embeddings", up(wl.tok)),
+        F("bert_embeddings_position_embeddings", up(wl.pos)), F("output_fp16", 1), F("mha_type_id", lib.F16),
+        F("eps", np.array([wl.eps], np.float32))])
+    e, midx = emb(dev(wl.input_ids), dev(wl.segment_ids), dev(wl.input_mask))
+    assert tuple(e.shape) == (64, 4, 1024, 1, 1) and tuple(midx.shape) == (4, 1) and e.dtype == torch.float16
+    wemb, wmidx, _ = oracle.emb_layer_norm(wl.input_ids, wl.segment_ids, wl.input_mask, wl.word, wl.pos, wl.tok,
+                                           wl.gamma, wl.beta, eps=wl.eps)
+    assert_close(host(e).reshape(64, 4, 1024), wemb, np.float16)
+    np.testing.assert_array_equal(host(midx).reshape(-1), wmidx)
+
+    cs = REG.getPluginCreator("CustomSkipLayerNormPluginDynamic", "1")
+    skip = cs.createPlugin("skip_ln", [F("beta", up(wl.skip_beta)), F("gamma", up(wl.skip_gamma)), F("ld", 1024),
+                                       F("type_id", lib.F16), F("bias", up(wl.skip_bias)),
+                                       F("eps", np.array([wl.eps], np.float32))])
+    res = dev(wl.skip.reshape(64, 4, 1024, 1, 1))
+    out = skip(e, res)
+    want = oracle.skip_layer_norm(host(e).reshape(64, 4, 1024), wl.skip_gamma, wl.skip_beta, skip=wl.skip,
+                                  bias=wl.skip_bias, eps=wl.eps)
+    assert_close(host(out).reshape(64, 4, 1024), want, np.float16)
+    # save / load keeps the result
+    out2 = cs.deserializePlugin("skip_ln", skip.serialize())(e, res)
+    np.testing.assert_array_equal(host(out), host(out2))
+    e2, _ = ce.deserializePlugin("embeddings", emb.serialize())(dev(wl.input_ids), dev(wl.segment_ids),
+                                                                dev(wl.input_mask))
+    np.testing.assert_array_equal(host(e), host(e2))
+    # a half-precision plugin refuses float input at configure time
+    with pytest.raises(lib.FwdmiError):
+        skip.configurePlugin([((64, 4, 1024), lib.F32)] * 2, [((64, 4, 1024), lib.F32)])

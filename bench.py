@@ -38,6 +38,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     ap.add_argument("--no-extra", action="store_true", help="skip the config 2/3/5 side measurements")
     ap.add_argument("--cpu-bags", type=int, default=4096, help="bags per table in the CPU baseline sample")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 1 GiB device-to-device copy (known traffic, to scale rocprof byte counters)")
     return ap.parse_args()
 
 
@@ -228,6 +230,13 @@ def main():
         with open(prof) as f:
             result["roofline"]["traffic"] = json.load(f).get("bag_reduce_config4_bytes_per_launch")
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)      # one elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     if not args.no_cpu:
         t1 = time.time()
         cpu, cpu_out, nb = cpu_baseline(wl, tabs, args.cpu_bags, torch)

@@ -33,7 +33,7 @@ constexpr int kIdxCap = 2048;      // ids staged in LDS per workgroup
 constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
 constexpr int kUnroll = 8;         // row loads in flight per lane
 
-enum Kind { kPlain = 0, kWeighted = 1, kMax = 2 };
+enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3 };
 
 struct BagLaunch {
   const fwdmi_bag_table* tables;  // device array, or nullptr -> `single`
@@ -61,6 +61,44 @@ struct alignas((sizeof(T) * N) < 16 ? (sizeof(T) * N) : 16) Pack {
   T v[N];
 };
 
+// Pointers that reach the kernel inside a struct (or are loaded from the table array) are
+// generic to the compiler, which then emits flat_* accesses; these casts pin them to global
+// memory so rows are fetched with global_load_dwordx4.
+#define FWDMI_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ const T FWDMI_GLOBAL* gconst(const void* p) {
+  return (const T FWDMI_GLOBAL*)(p);
+}
+template <typename T>
+__device__ __forceinline__ T FWDMI_GLOBAL* gmut(void* p) {
+  return (T FWDMI_GLOBAL*)(p);
+}
+
+// N-element (at most 16-byte aligned) vector load / store in global memory.
+template <typename T, int N>
+__device__ __forceinline__ Pack<T, N> gload(const T FWDMI_GLOBAL* p) {
+  Pack<T, N> r;
+  if constexpr (N == 1) {
+    r.v[0] = *p;
+  } else {
+    typedef T V __attribute__((ext_vector_type(N), aligned(alignof(Pack<T, N>))));
+    const V x = *(const V FWDMI_GLOBAL*)p;
+    __builtin_memcpy(&r, &x, sizeof(r));
+  }
+  return r;
+}
+template <typename T, int N>
+__device__ __forceinline__ void gstore(T FWDMI_GLOBAL* p, const Pack<T, N>& r) {
+  if constexpr (N == 1) {
+    *p = r.v[0];
+  } else {
+    typedef T V __attribute__((ext_vector_type(N), aligned(alignof(Pack<T, N>))));
+    V x;
+    __builtin_memcpy(&x, &r, sizeof(r));
+    *(V FWDMI_GLOBAL*)p = x;
+  }
+}
+
 template <typename TW, typename TI, int VEC, int KIND>
 __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
   __shared__ int64_t s_off[kMaxBagsPerWG + 1];
@@ -71,7 +109,19 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
   const int tid = threadIdx.x;
   const int t = blockIdx.x / L.wgs_per_table;
   const int wg = blockIdx.x - t * L.wgs_per_table;
-  const fwdmi_bag_table T = L.tables ? L.tables[t] : L.single;
+  fwdmi_bag_table T;
+  if (L.tables) {
+    const fwdmi_bag_table FWDMI_GLOBAL* tp = gconst<fwdmi_bag_table>(L.tables) + t;
+    T.data = tp->data;
+    T.input = tp->input;
+    T.input_2 = tp->input_2;
+    T.count = tp->count;
+    T.input_size = tp->input_size;
+    T.data_offset = tp->data_offset;
+    T.out_col = tp->out_col;
+  } else {
+    T = L.single;
+  }
 
   const int G = 1 << L.log2_g;
   const int slot = tid >> L.log2_g;
@@ -80,8 +130,8 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
 
   const int64_t bag0 = (int64_t)wg * L.bags_per_wg;
   const int nb = (int)min((int64_t)L.bags_per_wg, L.n_bags - bag0);
-  const TI* __restrict__ ids = static_cast<const TI*>(T.input);
-  const TW* __restrict__ psw = static_cast<const TW*>(L.psw);
+  const TI FWDMI_GLOBAL* __restrict__ ids = gconst<TI>(T.input);
+  const TW FWDMI_GLOBAL* __restrict__ psw = gconst<TW>(L.psw);
 
   // ---- stage the run's offsets (clamped) ------------------------------------------------
   for (int i = tid; i <= nb; i += kWG) {
@@ -90,8 +140,7 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
       v = (bag0 + i) * L.fixed_len;
     } else {
       const int64_t b = bag0 + i;
-      v = (b < L.n_bags || L.include_last) ? (int64_t) static_cast<const TI*>(T.input_2)[b]
-                                           : T.input_size;
+      v = (b < L.n_bags || L.include_last) ? (int64_t)gconst<TI>(T.input_2)[b] : T.input_size;
     }
     s_off[i] = min(max(v, (int64_t)0), T.input_size);
   }
@@ -110,9 +159,8 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
   }
   __syncthreads();
 
-  const TW* __restrict__ tab = static_cast<const TW*>(T.data);
+  const TW FWDMI_GLOBAL* __restrict__ tab = gconst<TW>(T.data);
   const int n_units = nb * L.n_slices;
-  const bool square = L.op == FWDMI_OP_SQUARE_SUM;
   bool oob = false;
 
   int unit = slot;
@@ -123,7 +171,7 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
     const int64_t end = max(s_off[lb + 1], start);
     const int col = (sl * G + gl) * VEC;
     const bool col_ok = col < L.dim;
-    const int col_c = col_ok ? col : 0;
+    const TW FWDMI_GLOBAL* __restrict__ tcol = tab + (col_ok ? col : 0);
     // A run whose offsets decrease can make [start,end) leave the staged window.
     const bool in_lds = staged && start >= span0 && end <= span0 + span;
 
@@ -135,33 +183,58 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
     for (int e = 0; e < (KIND == kMax ? VEC : 1); ++e) arg[e] = 0;
     bool first = true;
 
-    // Loads `UU` rows starting at bag position i, then folds them in order.
-    auto step = [&](auto uu_tag, int64_t i) {
+    // Loads UU rows starting at bag position i (all loads issued before the first use), then
+    // folds them in bag order.  LDS selects where the ids come from.
+    auto step = [&](auto uu_tag, auto lds_tag, int64_t i) {
       constexpr int UU = decltype(uu_tag)::value;
+      constexpr bool LDS = decltype(lds_tag)::value;
       Pack<TW, VEC> v[UU];
       TI id[UU];
       float w[UU];
       bool ok[UU];
+      bool all_ok = true;
 #pragma unroll
       for (int u = 0; u < UU; ++u) {
         const int64_t p = i + u;
-        id[u] = in_lds ? s_idx[p - span0] : ids[p];
-        if (KIND == kWeighted) w[u] = in_lds ? s_w[p - span0] : (float)psw[p];
+        if (LDS) {
+          id[u] = s_idx[(int)(p - span0)];
+          if (KIND == kWeighted) w[u] = s_w[(int)(p - span0)];
+        } else {
+          id[u] = ids[p];
+          if (KIND == kWeighted) w[u] = (float)psw[p];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UU; ++u) {
         const uint64_t row = (uint64_t)((int64_t)id[u] - T.data_offset);
         ok[u] = row < (uint64_t)T.count;
-        oob |= !ok[u];
+        all_ok &= ok[u];
         const uint64_t row_c = ok[u] ? row : 0;  // never form an address from a bad id
-        v[u] = *reinterpret_cast<const Pack<TW, VEC>*>(tab + row_c * (uint64_t)L.dim + col_c);
+        v[u] = gload<TW, VEC>(tcol + row_c * (uint64_t)L.dim);
+      }
+      if (__builtin_expect(!__all(all_ok), 0)) {
+        // rare: some id is out of range -> its row (row 0 was fetched instead) must not count
+        oob |= !all_ok;
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+          if (!ok[u]) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[u].v[e] = (TW)0.0f;
+            w[u] = 0.0f;
+          }
+        }
       }
 #pragma unroll
       for (int u = 0; u < UU; ++u) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          const float x = ok[u] ? (float)v[u].v[e] : 0.0f;
+          const float x = (float)v[u].v[e];
           if (KIND == kPlain) {
-            acc[e] = square ? __builtin_fmaf(x, x, acc[e]) : acc[e] + x;
+            acc[e] = acc[e] + x;
+          } else if (KIND == kSquare) {
+            acc[e] = __builtin_fmaf(x, x, acc[e]);
           } else if (KIND == kWeighted) {
-            acc[e] = __builtin_fmaf(ok[u] ? w[u] : 0.0f, x, acc[e]);
+            acc[e] = __builtin_fmaf(w[u], x, acc[e]);
           } else {
             if (ok[u] && (first || x > acc[e])) {
               acc[e] = x;
@@ -172,18 +245,23 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
         if (KIND == kMax && ok[u]) first = false;
       }
     };
-
-    int64_t i = start;
-    for (; i + kUnroll <= end; i += kUnroll) step(std::integral_constant<int, kUnroll>{}, i);
-    if (i + 4 <= end) {
-      step(std::integral_constant<int, 4>{}, i);
-      i += 4;
-    }
-    if (i + 2 <= end) {
-      step(std::integral_constant<int, 2>{}, i);
-      i += 2;
-    }
-    if (i < end) step(std::integral_constant<int, 1>{}, i);
+    auto bag = [&](auto lds_tag) {
+      int64_t i = start;
+      for (; i + kUnroll <= end; i += kUnroll) step(std::integral_constant<int, kUnroll>{}, lds_tag, i);
+      if (i + 4 <= end) {
+        step(std::integral_constant<int, 4>{}, lds_tag, i);
+        i += 4;
+      }
+      if (i + 2 <= end) {
+        step(std::integral_constant<int, 2>{}, lds_tag, i);
+        i += 2;
+      }
+      if (i < end) step(std::integral_constant<int, 1>{}, lds_tag, i);
+    };
+    if (in_lds)
+      bag(std::true_type{});
+    else
+      bag(std::false_type{});
 
     // ---- epilogue: mean scaling, store ---------------------------------------------------
     const int64_t len = end - start;
@@ -195,30 +273,30 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
     if (col_ok) {
       const int64_t o = (bag0 + lb) * L.out_stride + T.out_col + col;
       if (L.out_f16) {
-        _Float16* op = static_cast<_Float16*>(L.out) + o;
+        _Float16 FWDMI_GLOBAL* op = gmut<_Float16>(L.out) + o;
         if (L.vec_store) {
           Pack<_Float16, VEC> r;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) r.v[e] = (_Float16)acc[e];
-          *reinterpret_cast<Pack<_Float16, VEC>*>(op) = r;
+          gstore<_Float16, VEC>(op, r);
         } else {
 #pragma unroll
           for (int e = 0; e < VEC; ++e) op[e] = (_Float16)acc[e];
         }
       } else {
-        float* op = static_cast<float*>(L.out) + o;
+        float FWDMI_GLOBAL* op = gmut<float>(L.out) + o;
         if (L.vec_store) {
           Pack<float, VEC> r;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) r.v[e] = acc[e];
-          *reinterpret_cast<Pack<float, VEC>*>(op) = r;
+          gstore<float, VEC>(op, r);
         } else {
 #pragma unroll
           for (int e = 0; e < VEC; ++e) op[e] = acc[e];
         }
       }
       if (KIND == kMax && L.max_indices) {
-        TI* mp = static_cast<TI*>(L.max_indices) + (bag0 + lb) * (int64_t)L.dim + col;
+        TI FWDMI_GLOBAL* mp = gmut<TI>(L.max_indices) + (bag0 + lb) * (int64_t)L.dim + col;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) mp[e] = arg[e];
       }
@@ -238,6 +316,9 @@ int launch_kind(int kind, const BagLaunch& L, int grid, hipStream_t stream) {
   switch (kind) {
     case kPlain:
       hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kPlain>), dim3(grid), dim3(kWG), 0, stream, L);
+      break;
+    case kSquare:
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSquare>), dim3(grid), dim3(kWG), 0, stream, L);
       break;
     case kWeighted:
       hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kWeighted>), dim3(grid), dim3(kWG), 0, stream, L);
@@ -330,7 +411,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                 ((out_stride * so) % store_align) == 0 &&
                 (tables_dev || (single.out_col * so) % store_align == 0);
 
-  const int kind = op == FWDMI_OP_MAX ? kMax : (x.per_sample_weights ? kWeighted : kPlain);
+  const int kind = op == FWDMI_OP_MAX ? kMax : op == FWDMI_OP_SQUARE_SUM ? kSquare : (x.per_sample_weights ? kWeighted : kPlain);
   L.psw = x.per_sample_weights;
   const int grid = (int)(wgs * n_tables);
   const bool f16 = x.table_dtype == FWDMI_F16, i64 = x.index_dtype == FWDMI_I64;

@@ -10,8 +10,9 @@
 //   * A workgroup owns a contiguous run of bags.  Their offsets, and the ids (and weights)
 //     they cover, are copied into LDS once with coalesced loads; slots then read ids from
 //     LDS as broadcasts, so the only per-row global traffic is the row itself.
-//   * Slots pull the next bag of the run from an LDS counter, which evens out the long tail
-//     of bag lengths inside a workgroup.
+//   * The run's bags are ranked by length in LDS and handed out longest first from an LDS
+//     counter: the slots of a wavefront, which execute in lock-step, get bags of nearly equal
+//     length, and the long tail of bag lengths is evened out inside a workgroup.
 //   * Rows of one bag are added strictly in bag order (eight loads in flight, consumed in
 //     order), so fp32 results do not depend on the launch shape.
 //
@@ -21,6 +22,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <climits>
 #include <type_traits>
 
 #include "../common.h"
@@ -104,6 +106,8 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
   __shared__ int64_t s_off[kMaxBagsPerWG + 1];
   __shared__ TI s_idx[kIdxCap];
   __shared__ float s_w[KIND == kWeighted ? kIdxCap : 1];
+  __shared__ int s_len[kMaxBagsPerWG];
+  __shared__ uint16_t s_order[kMaxBagsPerWG];
   __shared__ int s_next;
 
   const int tid = threadIdx.x;
@@ -157,6 +161,25 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
       if (KIND == kWeighted) s_w[i] = (float)psw[span0 + i];
     }
   }
+  // ---- order the run's bags by length, longest first --------------------------------------
+  // The slots of one wavefront execute in lock-step, so a wavefront pays for the longest of
+  // the bags its slots hold.  Handing out bags in length order gives the slots of a wavefront
+  // bags of (nearly) equal length, and starting with the longest evens out the finish.
+  // The order changes which slot reduces a bag, never the result.
+  const bool sorted = L.fixed_len < 0 && nb > 1;
+  if (sorted) {
+    for (int i = tid; i < nb; i += kWG) s_len[i] = (int)min(max(s_off[i + 1] - s_off[i], (int64_t)0), (int64_t)INT_MAX);
+    __syncthreads();
+    for (int i = tid; i < nb; i += kWG) {
+      const int li = s_len[i];
+      int rank = 0;
+      for (int j = 0; j < nb; ++j) {
+        const int lj = s_len[j];
+        rank += (lj > li || (lj == li && j < i)) ? 1 : 0;
+      }
+      s_order[rank] = (uint16_t)i;
+    }
+  }
   __syncthreads();
 
   const TW FWDMI_GLOBAL* __restrict__ tab = gconst<TW>(T.data);
@@ -165,8 +188,9 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
 
   int unit = slot;
   while (unit < n_units) {
-    const int lb = L.n_slices == 1 ? unit : unit / L.n_slices;
-    const int sl = unit - lb * L.n_slices;
+    const int ub = L.n_slices == 1 ? unit : unit / L.n_slices;
+    const int sl = unit - ub * L.n_slices;
+    const int lb = sorted ? (int)s_order[ub] : ub;
     const int64_t start = s_off[lb];
     const int64_t end = max(s_off[lb + 1], start);
     const int col = (sl * G + gl) * VEC;

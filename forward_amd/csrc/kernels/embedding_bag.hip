@@ -56,6 +56,7 @@ struct BagLaunch {
   int32_t bags_per_wg;
   int32_t wgs_per_table;
   int32_t vec_store;
+  float one;  // 1.0f
 };
 
 template <typename T, int N>
@@ -184,7 +185,10 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
 
   const TW FWDMI_GLOBAL* __restrict__ tab = gconst<TW>(T.data);
   const int n_units = nb * L.n_slices;
+  // 32-bit id arithmetic is exact when ids are int32 and the table's id range lies in [0, 2^31).
+  const bool narrow = sizeof(TI) == 4 && T.data_offset >= 0 && T.data_offset + T.count <= ((int64_t)1 << 31);
   bool oob = false;
+  const float one = L.one;
 
   int unit = slot;
   while (unit < n_units) {
@@ -208,10 +212,12 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
     bool first = true;
 
     // Loads UU rows starting at bag position i (all loads issued before the first use), then
-    // folds them in bag order.  LDS selects where the ids come from.
-    auto step = [&](auto uu_tag, auto lds_tag, int64_t i) {
+    // folds them in bag order.  LDS selects where the ids come from; NARROW selects 32-bit id
+    // arithmetic (valid when every in-range id is a non-negative int32).
+    auto step = [&](auto uu_tag, auto lds_tag, auto narrow_tag, int64_t i) {
       constexpr int UU = decltype(uu_tag)::value;
       constexpr bool LDS = decltype(lds_tag)::value;
+      constexpr bool NARROW = decltype(narrow_tag)::value;
       Pack<TW, VEC> v[UU];
       TI id[UU];
       float w[UU];
@@ -230,14 +236,19 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
       }
 #pragma unroll
       for (int u = 0; u < UU; ++u) {
-        const uint64_t row = (uint64_t)((int64_t)id[u] - T.data_offset);
-        ok[u] = row < (uint64_t)T.count;
+        // a bad id never forms an address: row 0 is fetched instead and discarded below
+        if (NARROW) {
+          const uint32_t row = (uint32_t)id[u] - (uint32_t)T.data_offset;
+          ok[u] = row < (uint32_t)T.count;
+          v[u] = gload<TW, VEC>(tcol + (uint64_t)(ok[u] ? row : 0u) * (uint32_t)L.dim);
+        } else {
+          const uint64_t row = (uint64_t)((int64_t)id[u] - T.data_offset);
+          ok[u] = row < (uint64_t)T.count;
+          v[u] = gload<TW, VEC>(tcol + (ok[u] ? row : 0) * (uint64_t)L.dim);
+        }
         all_ok &= ok[u];
-        const uint64_t row_c = ok[u] ? row : 0;  // never form an address from a bad id
-        v[u] = gload<TW, VEC>(tcol + row_c * (uint64_t)L.dim);
       }
       if (__builtin_expect(!__all(all_ok), 0)) {
-        // rare: some id is out of range -> its row (row 0 was fetched instead) must not count
         oob |= !all_ok;
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
@@ -254,7 +265,10 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
         for (int e = 0; e < VEC; ++e) {
           const float x = (float)v[u].v[e];
           if (KIND == kPlain) {
-            acc[e] = acc[e] + x;
+            // fma(x, 1, acc) rounds exactly like acc + x and lets fp16 rows use the
+            // mixed-precision FMA (conversion and add in one instruction); `one` arrives as a
+            // kernel argument so the multiply is not folded away
+            acc[e] = __builtin_fmaf(x, one, acc[e]);
           } else if (KIND == kSquare) {
             acc[e] = __builtin_fmaf(x, x, acc[e]);
           } else if (KIND == kWeighted) {
@@ -269,23 +283,27 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
         if (KIND == kMax && ok[u]) first = false;
       }
     };
-    auto bag = [&](auto lds_tag) {
+    auto bag = [&](auto lds_tag, auto narrow_tag) {
       int64_t i = start;
-      for (; i + kUnroll <= end; i += kUnroll) step(std::integral_constant<int, kUnroll>{}, lds_tag, i);
+      for (; i + kUnroll <= end; i += kUnroll) step(std::integral_constant<int, kUnroll>{}, lds_tag, narrow_tag, i);
       if (i + 4 <= end) {
-        step(std::integral_constant<int, 4>{}, lds_tag, i);
+        step(std::integral_constant<int, 4>{}, lds_tag, narrow_tag, i);
         i += 4;
       }
       if (i + 2 <= end) {
-        step(std::integral_constant<int, 2>{}, lds_tag, i);
+        step(std::integral_constant<int, 2>{}, lds_tag, narrow_tag, i);
         i += 2;
       }
-      if (i < end) step(std::integral_constant<int, 1>{}, lds_tag, i);
+      if (i < end) step(std::integral_constant<int, 1>{}, lds_tag, narrow_tag, i);
     };
-    if (in_lds)
-      bag(std::true_type{});
-    else
-      bag(std::false_type{});
+    if (in_lds) {
+      if (narrow)
+        bag(std::true_type{}, std::true_type{});
+      else
+        bag(std::true_type{}, std::false_type{});
+    } else {
+      bag(std::false_type{}, std::false_type{});
+    }
 
     // ---- epilogue: mean scaling, store ---------------------------------------------------
     const int64_t len = end - start;
@@ -415,6 +433,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   L.n_bags = n_bags;
   L.out_stride = out_stride;
   L.fixed_len = fixed_len;
+  L.one = 1.0f;
   L.dim = dim;
   L.op = op;
   L.out_f16 = x.out_dtype == FWDMI_F16;

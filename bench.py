@@ -35,6 +35,7 @@ def parse():
     ap.add_argument("--tables", type=int, default=26, help="debug only: fewer tables (not the named config)")
     ap.add_argument("--bags", type=int, default=65536, help="debug only: smaller batch (not the named config)")
     ap.add_argument("--per-table", action="store_true", help="26 launches instead of the fused one")
+    ap.add_argument("--xcd-affinity", action="store_true", help="fused launch with per-XCD table affinity")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     ap.add_argument("--no-extra", action="store_true", help="skip the config 2/3/5 side measurements")
     ap.add_argument("--cpu-bags", type=int, default=4096, help="bags per table in the CPU baseline sample")
@@ -197,7 +198,7 @@ def main():
         launches_per_step = batch.n_tables
     else:
         def step():
-            batch.forward(out=out)
+            batch.forward(out=out, xcd_table_affinity=args.xcd_affinity)
         launches_per_step = 1
 
     wall, per = time_events(torch, step, args.steps, args.warmup)

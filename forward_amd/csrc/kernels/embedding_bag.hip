@@ -31,9 +31,18 @@ namespace fwdmi {
 namespace {
 
 constexpr int kWG = 256;           // lanes per workgroup
-constexpr int kIdxCap = 2048;      // ids staged in LDS per workgroup
+constexpr int kIdxBytes = 16384;   // LDS bytes for staged ids per workgroup (4096 int32 / 2048 int64)
+constexpr int kXcds = 8;           // accelerator complex dies; workgroup b is dispatched to XCD b % 8
 constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
-constexpr int kUnroll = 8;         // row loads in flight per lane
+#ifndef FWDMI_BAG_UNROLL
+#define FWDMI_BAG_UNROLL 8
+#endif
+#ifdef FWDMI_BAG_WAVES_PER_EU
+#define FWDMI_BAG_OCCUPANCY __attribute__((amdgpu_waves_per_eu(FWDMI_BAG_WAVES_PER_EU)))
+#else
+#define FWDMI_BAG_OCCUPANCY
+#endif
+constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 
 enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3 };
 
@@ -57,6 +66,8 @@ struct BagLaunch {
   int32_t wgs_per_table;
   int32_t vec_store;
   float one;  // 1.0f
+  int32_t xcd_chunk;  // > 0: workgroups are renumbered so each XCD owns a contiguous range of tables
+  int32_t total_wgs;
 };
 
 template <typename T, int N>
@@ -103,8 +114,9 @@ __device__ __forceinline__ void gstore(T FWDMI_GLOBAL* p, const Pack<T, N>& r) {
 }
 
 template <typename TW, typename TI, int VEC, int KIND>
-__global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
+__global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(const BagLaunch L) {
   __shared__ int64_t s_off[kMaxBagsPerWG + 1];
+  constexpr int kIdxCap = kIdxBytes / sizeof(TI);
   __shared__ TI s_idx[kIdxCap];
   __shared__ float s_w[KIND == kWeighted ? kIdxCap : 1];
   __shared__ int s_len[kMaxBagsPerWG];
@@ -112,8 +124,16 @@ __global__ __launch_bounds__(kWG) void bag_reduce_kernel(const BagLaunch L) {
   __shared__ int s_next;
 
   const int tid = threadIdx.x;
-  const int t = blockIdx.x / L.wgs_per_table;
-  const int wg = blockIdx.x - t * L.wgs_per_table;
+  // Each XCD has its own L2.  On request, a multi-table launch undoes the hardware's round-robin
+  // placement (workgroup b runs on XCD b % 8) so that one XCD works through whole tables: a
+  // table's hot rows are then fetched into one L2 instead of all eight.
+  int work = blockIdx.x;
+  if (L.xcd_chunk > 0) {
+    work = (int)(blockIdx.x % kXcds) * L.xcd_chunk + (int)(blockIdx.x / kXcds);
+    if (work >= L.total_wgs) return;
+  }
+  const int t = work / L.wgs_per_table;
+  const int wg = work - t * L.wgs_per_table;
   fwdmi_bag_table T;
   if (L.tables) {
     const fwdmi_bag_table FWDMI_GLOBAL* tp = gconst<fwdmi_bag_table>(L.tables) + t;
@@ -391,7 +411,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                  void* output, int64_t n_bags, int64_t fixed_len, int dim, int op, double avg_len,
                  const fwdmi_bag_ext* ext, hipStream_t stream) {
   clear_error();
-  static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr};
+  static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0};
   const fwdmi_bag_ext& x = ext ? *ext : kDefaultExt;
 
   if (!is_float_dtype(x.table_dtype) || !is_float_dtype(x.out_dtype) || !is_index_dtype(x.index_dtype))
@@ -443,8 +463,9 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   L.n_slices = (dim + lanes * VEC - 1) / (lanes * VEC);
   const int slots = kWG / lanes;
   if (avg_len < 1.0) avg_len = 1.0;
-  int k = (int)(kIdxCap / 1.5 / (avg_len * slots));
-  k = std::max(1, std::min(8, k));
+  const int idx_cap = kIdxBytes / (int)dtype_size(x.index_dtype);
+  int k = (int)(idx_cap / 1.5 / (avg_len * slots));
+  k = std::max(1, std::min(16, k));
   L.bags_per_wg = std::max(1, std::min(kMaxBagsPerWG, slots * k / L.n_slices));
   const int64_t wgs = (n_bags + L.bags_per_wg - 1) / L.bags_per_wg;
   FWDMI_REQUIRE(wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
@@ -456,7 +477,13 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
 
   const int kind = op == FWDMI_OP_MAX ? kMax : op == FWDMI_OP_SQUARE_SUM ? kSquare : (x.per_sample_weights ? kWeighted : kPlain);
   L.psw = x.per_sample_weights;
-  const int grid = (int)(wgs * n_tables);
+  int grid = (int)(wgs * n_tables);
+  L.total_wgs = grid;
+  L.xcd_chunk = 0;
+  if (tables_dev && n_tables > 1 && (x.flags & FWDMI_BAG_XCD_TABLE_AFFINITY)) {
+    L.xcd_chunk = (grid + kXcds - 1) / kXcds;
+    grid = L.xcd_chunk * kXcds;
+  }
   const bool f16 = x.table_dtype == FWDMI_F16, i64 = x.index_dtype == FWDMI_I64;
   if (f16)
     return i64 ? launch_vec<_Float16, int64_t>(vec, kind, L, grid, stream)
@@ -496,7 +523,7 @@ int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t of
     return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "gather: batch %lld x %lld", (long long)batch_size,
                             (long long)offset);
   // A gather is a sum over bags of exactly one id.
-  fwdmi_bag_ext x = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr};
+  fwdmi_bag_ext x = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0};
   x.per_sample_weights = nullptr;
   x.max_indices = nullptr;
   x.out_row_stride = 0;

@@ -19,6 +19,7 @@ const fwdmi_bag_ext make_ext(const EmbeddingBagOptions& o, const void* psw, int3
   x.max_indices = nullptr;
   x.out_row_stride = 0;
   x.oob_flag = oob;
+  x.flags = 0;
   return x;
 }
 

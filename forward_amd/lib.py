@@ -23,12 +23,14 @@ F32, F16, I8, I32, BOOL, I64 = 0, 1, 2, 3, 4, 10
 FIELD_F16, FIELD_F32, FIELD_F64, FIELD_I8, FIELD_I16, FIELD_I32, FIELD_CHAR, FIELD_DIMS, FIELD_UNKNOWN = range(9)
 FORMAT_LINEAR = 0
 OP_SUM, OP_MEAN, OP_MAX, OP_SQUARE_SUM, OP_GATHER = 0, 1, 2, 3, 999
+BAG_XCD_TABLE_AFFINITY = 1
 
 
 class BagExt(C.Structure):
     _fields_ = [("table_dtype", C.c_int32), ("index_dtype", C.c_int32), ("out_dtype", C.c_int32),
                 ("include_last_offset", C.c_int32), ("per_sample_weights", C.c_void_p),
-                ("max_indices", C.c_void_p), ("out_row_stride", C.c_int64), ("oob_flag", C.c_void_p)]
+                ("max_indices", C.c_void_p), ("out_row_stride", C.c_int64), ("oob_flag", C.c_void_p),
+                ("flags", C.c_int32)]
 
 
 class BagTable(C.Structure):

@@ -38,7 +38,7 @@ def _op(mode):
 
 
 def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_indices=None, out_row_stride=0,
-         oob_flag=None):
+         oob_flag=None, flags=0):
     x = lib.BagExt()
     x.table_dtype = _FDT[table.dtype]
     x.index_dtype = _IDT[indices.dtype]
@@ -48,6 +48,7 @@ def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_ind
     x.max_indices = max_indices.data_ptr() if max_indices is not None else None
     x.out_row_stride = int(out_row_stride)
     x.oob_flag = oob_flag.data_ptr() if oob_flag is not None else None
+    x.flags = flags
     return x
 
 
@@ -140,13 +141,14 @@ class MultiTableBatch:
         self.total_indices = int(sum(i.numel() for i in self.indices))
         self.desc = torch.from_numpy(desc).to(self.tables[0].device)
 
-    def forward(self, out=None, mode="sum", out_dtype=None, oob_flag=None, stream=None):
+    def forward(self, out=None, mode="sum", out_dtype=None, oob_flag=None, xcd_table_affinity=False, stream=None):
         odt = self.tables[0].dtype if out_dtype is None else out_dtype
         if out is None:
             out = torch.empty((self.n_bags, self.width), dtype=odt, device=self.desc.device)
         _dev(out, "out")
         assert out.dtype == odt and out.shape[0] == self.n_bags and out.shape[1] >= self.width
-        x = _ext(self.tables[0], self.indices[0], odt, out_row_stride=out.shape[1], oob_flag=oob_flag)
+        x = _ext(self.tables[0], self.indices[0], odt, out_row_stride=out.shape[1], oob_flag=oob_flag,
+                 flags=lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0)
         avg = self.total_indices / max(1, self.n_bags * self.n_tables)
         lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(self.desc), self.n_tables, self.n_bags, _p(out), self.dim,
                                                     _op(mode), avg, C.byref(x), _stream(stream)))

@@ -86,7 +86,13 @@ typedef struct fwdmi_bag_ext {
                                   write column blocks of one concatenated matrix) */
   int32_t* oob_flag;           /* device int, set to 1 (sticky) when an id falls outside
                                   [data_offset, data_offset+count); may be NULL */
+  int32_t flags;               /* FWDMI_BAG_* bits, 0 for none */
 } fwdmi_bag_ext;
+
+/* Multi-table launches only: renumber workgroups so that each of the 8 XCDs (one L2 each)
+ * works through whole tables.  Cuts L2 fill traffic; off by default because on the 26-table
+ * configuration the uneven per-table cost outweighs it. */
+#define FWDMI_BAG_XCD_TABLE_AFFINITY 1
 
 /*
  * Variable-length bags: bag b = input[input_2[b] .. input_2[b+1]), last bag ends at input_size.

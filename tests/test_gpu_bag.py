@@ -156,6 +156,7 @@ def test_multi_table_concatenated(oracle):
     for t in range(5):
         ops.embedding_bag(batch.tables[t], batch.indices[t], batch.offsets[t], "sum", out=out, out_col=128 * t)
     assert_bits_equal(host(out), want, "per-table launches")
+    assert_bits_equal(host(batch.forward(xcd_table_affinity=True)), want, "fused, per-XCD table affinity")
     got32 = host(batch.forward(out_dtype=torch.float32))
     np.testing.assert_allclose(got32, want.astype(np.float32), atol=1e-2, rtol=5e-3)
 

@@ -46,13 +46,7 @@ def parse():
 
 def device_tables(wl, torch):
     """fp16 rows ~U(-0.05, 0.05) generated in HBM (seeded per table)."""
-    tabs = []
-    for t, rows in enumerate(wl.rows):
-        g = torch.Generator(device="cuda").manual_seed(wl.table_seeds[t])
-        x = torch.rand((rows, wl.dim), generator=g, device="cuda", dtype=torch.float32)
-        tabs.append(((x - 0.5) * 0.1).to(torch.float16))
-        del x
-    return tabs
+    return [wl.device_table(t, torch) for t in range(len(wl.rows))]
 
 
 def time_events(torch, fn, steps, warmup):

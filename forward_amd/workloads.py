@@ -180,6 +180,13 @@ class MultiTableWorkload:
         return (n * (self.dim * table_itemsize + index_itemsize) + t * self.n_bags * index_itemsize
                 + t * self.n_bags * self.dim * out_itemsize)
 
+    def device_table(self, t, torch):
+        """Rows ~U(-0.05, 0.05) of table ``t`` as fp16, generated directly in HBM (seeded per
+        table; a different stream of values than ``host_table``, for full-size runs)."""
+        g = torch.Generator(device="cuda").manual_seed(self.table_seeds[t])
+        x = torch.rand((self.rows[t], self.dim), generator=g, device="cuda", dtype=torch.float32)
+        return ((x - 0.5) * 0.1).to(torch.float16)
+
     def host_table(self, t, dtype=np.float16):
         """Rows ~U(-0.05, 0.05) of table ``t`` (own seed, so tables can be made one at a time)."""
         rng = np.random.Generator(np.random.PCG64(self.table_seeds[t]))

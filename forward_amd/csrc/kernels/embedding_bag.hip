@@ -30,7 +30,7 @@
 namespace fwdmi {
 namespace {
 
-constexpr int kWG = 256;           // lanes per workgroup
+constexpr int kWG = 256;           // lanes per workgroup (large batches; small ones use 128 or 64)
 constexpr int kIdxBytes = 16384;   // LDS bytes for staged ids per workgroup (4096 int32 / 2048 int64)
 constexpr int kXcds = 8;           // accelerator complex dies; workgroup b is dispatched to XCD b % 8
 constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
@@ -68,6 +68,7 @@ struct BagLaunch {
   float one;  // 1.0f
   int32_t xcd_chunk;  // > 0: workgroups are renumbered so each XCD owns a contiguous range of tables
   int32_t total_wgs;
+  int32_t idx_cap;    // ids the LDS window holds
 };
 
 template <typename T, int N>
@@ -115,13 +116,16 @@ __device__ __forceinline__ void gstore(T FWDMI_GLOBAL* p, const Pack<T, N>& r) {
 
 template <typename TW, typename TI, int VEC, int KIND>
 __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(const BagLaunch L) {
-  __shared__ int64_t s_off[kMaxBagsPerWG + 1];
-  constexpr int kIdxCap = kIdxBytes / sizeof(TI);
-  __shared__ TI s_idx[kIdxCap];
-  __shared__ float s_w[KIND == kWeighted ? kIdxCap : 1];
-  __shared__ int s_len[kMaxBagsPerWG];
-  __shared__ uint16_t s_order[kMaxBagsPerWG];
+  // LDS carve-up (dynamic, sized by the host): offsets | ids | weights | lengths | order
+  extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
+  int64_t* const s_off = reinterpret_cast<int64_t*>(s_raw);
+  TI* const s_idx = reinterpret_cast<TI*>(s_off + (L.bags_per_wg + 2));
+  float* const s_w = reinterpret_cast<float*>(s_idx + L.idx_cap);
+  int* const s_len = reinterpret_cast<int*>(s_w + (KIND == kWeighted ? L.idx_cap : 0));
+  uint16_t* const s_order = reinterpret_cast<uint16_t*>(s_len + L.bags_per_wg);
   __shared__ int s_next;
+  const int kIdxCap = L.idx_cap;
+  const int wg_lanes = blockDim.x;
 
   const int tid = threadIdx.x;
   // Each XCD has its own L2.  On request, a multi-table launch undoes the hardware's round-robin
@@ -151,7 +155,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const int G = 1 << L.log2_g;
   const int slot = tid >> L.log2_g;
   const int gl = tid & (G - 1);
-  const int slots = kWG >> L.log2_g;
+  const int slots = wg_lanes >> L.log2_g;
 
   const int64_t bag0 = (int64_t)wg * L.bags_per_wg;
   const int nb = (int)min((int64_t)L.bags_per_wg, L.n_bags - bag0);
@@ -159,7 +163,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const TW FWDMI_GLOBAL* __restrict__ psw = gconst<TW>(L.psw);
 
   // ---- stage the run's offsets (clamped) ------------------------------------------------
-  for (int i = tid; i <= nb; i += kWG) {
+  for (int i = tid; i <= nb; i += wg_lanes) {
     int64_t v;
     if (L.fixed_len >= 0) {
       v = (bag0 + i) * L.fixed_len;
@@ -177,7 +181,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const int64_t span = s_off[nb] - span0;
   const bool staged = span >= 0 && span <= kIdxCap;  // uniform over the workgroup
   if (staged) {
-    for (int i = tid; i < span; i += kWG) {
+    for (int i = tid; i < span; i += wg_lanes) {
       s_idx[i] = ids[span0 + i];
       if (KIND == kWeighted) s_w[i] = (float)psw[span0 + i];
     }
@@ -189,9 +193,9 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   // The order changes which slot reduces a bag, never the result.
   const bool sorted = L.fixed_len < 0 && nb > 1;
   if (sorted) {
-    for (int i = tid; i < nb; i += kWG) s_len[i] = (int)min(max(s_off[i + 1] - s_off[i], (int64_t)0), (int64_t)INT_MAX);
+    for (int i = tid; i < nb; i += wg_lanes) s_len[i] = (int)min(max(s_off[i + 1] - s_off[i], (int64_t)0), (int64_t)INT_MAX);
     __syncthreads();
-    for (int i = tid; i < nb; i += kWG) {
+    for (int i = tid; i < nb; i += wg_lanes) {
       const int li = s_len[i];
       int rank = 0;
       for (int j = 0; j < nb; ++j) {
@@ -373,30 +377,55 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   if (oob && L.oob_flag) atomicOr(L.oob_flag, 1);
 }
 
+struct BagShape {
+  int grid, block;
+  size_t lds;
+};
+
+// Bytes of the kernel's LDS carve-up.
+size_t bag_lds_bytes(const BagLaunch& L, size_t index_size, bool weighted) {
+  size_t b = (size_t)(L.bags_per_wg + 2) * sizeof(int64_t) + (size_t)L.idx_cap * index_size;
+  if (weighted) b += (size_t)L.idx_cap * sizeof(float);
+  b += (size_t)L.bags_per_wg * (sizeof(int) + sizeof(uint16_t));
+  return (b + 15) & ~(size_t)15;
+}
+
 template <typename TW, typename TI, int VEC>
-int launch_kind(int kind, const BagLaunch& L, int grid, hipStream_t stream) {
+int launch_kind(int kind, const BagLaunch& L, const BagShape& sh, hipStream_t stream) {
+  const dim3 grid(sh.grid), block(sh.block);
   switch (kind) {
     case kPlain:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kPlain>), dim3(grid), dim3(kWG), 0, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kPlain>), grid, block, sh.lds, stream, L);
       break;
     case kSquare:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSquare>), dim3(grid), dim3(kWG), 0, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSquare>), grid, block, sh.lds, stream, L);
       break;
     case kWeighted:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kWeighted>), dim3(grid), dim3(kWG), 0, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kWeighted>), grid, block, sh.lds, stream, L);
       break;
     default:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMax>), dim3(grid), dim3(kWG), 0, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMax>), grid, block, sh.lds, stream, L);
   }
   FWDMI_HIP_CHECK(hipGetLastError());
   return FWDMI_OK;
 }
 
 template <typename TW, typename TI>
-int launch_vec(bool vec, int kind, const BagLaunch& L, int grid, hipStream_t stream) {
+int launch_vec(bool vec, int kind, const BagLaunch& L, const BagShape& sh, hipStream_t stream) {
   constexpr int kVec = 16 / sizeof(TW);
-  return vec ? launch_kind<TW, TI, kVec>(kind, L, grid, stream)
-             : launch_kind<TW, TI, 1>(kind, L, grid, stream);
+  return vec ? launch_kind<TW, TI, kVec>(kind, L, sh, stream)
+             : launch_kind<TW, TI, 1>(kind, L, sh, stream);
+}
+
+int device_cus() {
+  static const int cus = [] {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      return v;
+    return 256;
+  }();
+  return cus;
 }
 
 int next_pow2(int v) {
@@ -461,12 +490,23 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   const int lanes = std::min(64, next_pow2((dim + VEC - 1) / VEC));
   L.log2_g = __builtin_ctz(lanes);
   L.n_slices = (dim + lanes * VEC - 1) / (lanes * VEC);
-  const int slots = kWG / lanes;
   if (avg_len < 1.0) avg_len = 1.0;
-  const int idx_cap = kIdxBytes / (int)dtype_size(x.index_dtype);
-  int k = (int)(idx_cap / 1.5 / (avg_len * slots));
-  k = std::max(1, std::min(16, k));
-  L.bags_per_wg = std::max(1, std::min(kMaxBagsPerWG, slots * k / L.n_slices));
+  // Run length: as many bags as keep the run's ids inside the LDS window, but no more than leaves
+  // the chip with ~4 workgroups per CU; small batches also shrink the workgroup (down to one
+  // wavefront) so that every CU gets work.
+  const int max_cap = kIdxBytes / (int)dtype_size(x.index_dtype);
+  const int64_t total_bags = n_bags * n_tables;
+  const int64_t target_wgs = (int64_t)device_cus() * 4;
+  int64_t want_bags = std::max<int64_t>(1, total_bags / target_wgs);
+  const int64_t fit_bags = std::max<int64_t>(1, (int64_t)(max_cap / 1.5 / avg_len));
+  want_bags = std::min<int64_t>(std::min(want_bags, fit_bags), kMaxBagsPerWG);
+  int block = kWG;
+  while (block > 64 && block / 2 >= lanes && (int64_t)(block / 2 / lanes) * 4 >= want_bags * L.n_slices) block /= 2;
+  const int slots = block / lanes;
+  // a whole number of rounds over the slots
+  int64_t units = std::max<int64_t>(slots, want_bags * L.n_slices / slots * slots);
+  L.bags_per_wg = (int)std::max<int64_t>(1, std::min<int64_t>(kMaxBagsPerWG, units / L.n_slices));
+  L.idx_cap = std::min(max_cap, std::max(64, next_pow2((int)std::min<double>(max_cap, avg_len * L.bags_per_wg * 2.0))));
   const int64_t wgs = (n_bags + L.bags_per_wg - 1) / L.bags_per_wg;
   FWDMI_REQUIRE(wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
   L.wgs_per_table = (int)wgs;
@@ -485,11 +525,12 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
     grid = L.xcd_chunk * kXcds;
   }
   const bool f16 = x.table_dtype == FWDMI_F16, i64 = x.index_dtype == FWDMI_I64;
+  const BagShape sh{grid, block, bag_lds_bytes(L, dtype_size(x.index_dtype), kind == kWeighted)};
   if (f16)
-    return i64 ? launch_vec<_Float16, int64_t>(vec, kind, L, grid, stream)
-               : launch_vec<_Float16, int32_t>(vec, kind, L, grid, stream);
-  return i64 ? launch_vec<float, int64_t>(vec, kind, L, grid, stream)
-             : launch_vec<float, int32_t>(vec, kind, L, grid, stream);
+    return i64 ? launch_vec<_Float16, int64_t>(vec, kind, L, sh, stream)
+               : launch_vec<_Float16, int32_t>(vec, kind, L, sh, stream);
+  return i64 ? launch_vec<float, int64_t>(vec, kind, L, sh, stream)
+             : launch_vec<float, int32_t>(vec, kind, L, sh, stream);
 }
 
 }  // namespace

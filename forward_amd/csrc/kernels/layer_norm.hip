@@ -14,10 +14,14 @@
 #include <algorithm>
 
 #include "../common.h"
+#include "device_util.h"
 
 namespace fwdmi {
 namespace {
 
+#ifndef FWDMI_LN_BLOCKS_PER_CU
+#define FWDMI_LN_BLOCKS_PER_CU 8
+#endif
 constexpr int kWG = 256;
 constexpr int kWavesPerWG = kWG / 64;
 
@@ -44,11 +48,6 @@ struct LnLaunch {
   int32_t row_blocks;  // workgroups that process rows; the rest compute mask indices
   int32_t total_waves; // row-processing wavefronts in the grid
   float eps;
-};
-
-template <typename T, int N>
-struct alignas((sizeof(T) * N) < 16 ? (sizeof(T) * N) : 16) Pack {
-  T v[N];
 };
 
 struct Welford {
@@ -112,6 +111,15 @@ __device__ __forceinline__ void mask_index_wave(const LnLaunch& L, int b, int la
   if (lane == 0) L.mask_idx[b] = first;
 }
 
+// Register image of one row's operands: up to three 16-byte slices per chunk.
+template <typename T, int VEC, int NV, int MODE>
+struct RowRegs {
+  Pack<T, VEC> a[NV];                        // input / word row
+  Pack<T, VEC> b[MODE == kLayerNorm ? 1 : NV];  // skip / position row
+  Pack<T, VEC> c[MODE == kEmb ? NV : 1];     // token-type row
+  bool ok0, ok1, ok2;
+};
+
 template <typename T, int VEC, int NV, int MODE>
 __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   const int lane = threadIdx.x & 63;
@@ -124,75 +132,89 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
     return;
   }
   const int wave = blockIdx.x * kWavesPerWG + wave_in_wg;
+  const T FWDMI_GLOBAL* const in0 = gconst<T>(L.input);
+  const T FWDMI_GLOBAL* const in1 = gconst<T>(MODE == kEmb ? L.pos : L.skip);
+  const T FWDMI_GLOBAL* const in2 = gconst<T>(L.tok);
+  const int32_t FWDMI_GLOBAL* const ids = gconst<int32_t>(L.input_ids);
+  const int32_t FWDMI_GLOBAL* const segs = gconst<int32_t>(L.segment_ids);
 
   // Per-lane column slices: chunk j covers elements (j*64 + lane)*VEC .. +VEC.
   bool live[NV];
-  float g[NV][VEC], be[NV][VEC], bi[NV][VEC];
+  int col[NV];
   float cnt = 0.0f;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int c = (j * 64 + lane) * VEC;
     live[j] = c < L.ld;
-    const int cc = live[j] ? c : 0;
-    const Pack<float, VEC> pg = *reinterpret_cast<const Pack<float, VEC>*>(L.gamma + cc);
-    const Pack<float, VEC> pb = *reinterpret_cast<const Pack<float, VEC>*>(L.beta + cc);
+    col[j] = live[j] ? c : 0;
+    if (live[j]) cnt += (float)VEC;
+  }
+  const float inv_cnt = cnt > 0.0f ? 1.0f / cnt : 0.0f;
+
+  using Regs = RowRegs<T, VEC, NV, MODE>;
+  // Issues the loads of row r (no use of the data yet).
+  auto fetch = [&](int64_t r, Regs& R) {
+    if (MODE == kEmb) {
+      const int s = (int)(r / L.B);
+      const int64_t w = ids[r], sg = segs[r];
+      R.ok0 = w >= 0 && w < L.word_count;
+      R.ok1 = s < L.pos_count;
+      R.ok2 = sg >= 0 && sg < L.tok_count;
+      const T FWDMI_GLOBAL* wp = in0 + (R.ok0 ? w : 0) * L.ld;
+      const T FWDMI_GLOBAL* pp = in1 + (int64_t)(R.ok1 ? s : 0) * L.ld;
+      const T FWDMI_GLOBAL* tp = in2 + (R.ok2 ? sg : 0) * L.ld;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        R.a[j] = gload<T, VEC>(wp + col[j]);
+        R.b[j] = gload<T, VEC>(pp + col[j]);
+        R.c[j] = gload<T, VEC>(tp + col[j]);
+      }
+    } else {
+      R.ok0 = R.ok1 = R.ok2 = true;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        R.a[j] = gload<T, VEC>(in0 + r * L.ld + col[j]);
+        if (MODE == kSkip) R.b[j] = gload<T, VEC>(in1 + r * L.ld + col[j]);
+      }
+    }
+  };
+
+  // gamma / beta / bias stay in registers for every row this wavefront handles.
+  float g[NV][VEC], be[NV][VEC], bi[NV][VEC];
+  Regs cur, nxt;
+  int64_t r = wave;
+  if (r < L.rows) fetch(r, cur);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const Pack<float, VEC> pg = gload<float, VEC>(gconst<float>(L.gamma) + col[j]);
+    const Pack<float, VEC> pb = gload<float, VEC>(gconst<float>(L.beta) + col[j]);
     Pack<float, VEC> pi{};
-    if (L.bias) pi = *reinterpret_cast<const Pack<float, VEC>*>(L.bias + cc);
+    if (L.bias) pi = gload<float, VEC>(gconst<float>(L.bias) + col[j]);
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
       g[j][e] = pg.v[e];
       be[j][e] = pb.v[e];
       bi[j][e] = L.bias ? pi.v[e] : 0.0f;
     }
-    if (live[j]) cnt += (float)VEC;
   }
-  const float inv_cnt = cnt > 0.0f ? 1.0f / cnt : 0.0f;
 
   bool oob = false;
-  for (int64_t r = wave; r < L.rows; r += L.total_waves) {
+  for (; r < L.rows; r += L.total_waves) {
+    // the next row's loads are in flight while this row is reduced
+    const int64_t rn = r + L.total_waves;
+    if (rn < L.rows) fetch(rn, nxt);
+
     float x[NV][VEC];
-    if (MODE == kEmb) {
-      const int s = (int)(r / L.B);
-      const int64_t w = L.input_ids[r], sg = L.segment_ids[r];
-      const bool wok = w >= 0 && w < L.word_count, gok = sg >= 0 && sg < L.tok_count,
-                 pok = s < L.pos_count;
-      oob |= !(wok && gok && pok);
-      const T* wp = static_cast<const T*>(L.input) + (wok ? w : 0) * L.ld;
-      const T* pp = static_cast<const T*>(L.pos) + (int64_t)(pok ? s : 0) * L.ld;
-      const T* tp = static_cast<const T*>(L.tok) + (gok ? sg : 0) * L.ld;
-      Pack<T, VEC> a[NV], p[NV], q[NV];
+    if (MODE == kEmb) oob |= !(cur.ok0 && cur.ok1 && cur.ok2);
 #pragma unroll
-      for (int j = 0; j < NV; ++j) {
-        const int cc = live[j] ? (j * 64 + lane) * VEC : 0;
-        a[j] = *reinterpret_cast<const Pack<T, VEC>*>(wp + cc);
-        p[j] = *reinterpret_cast<const Pack<T, VEC>*>(pp + cc);
-        q[j] = *reinterpret_cast<const Pack<T, VEC>*>(tp + cc);
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float v = cur.ok0 ? (float)cur.a[j].v[e] : 0.0f;
+        if (MODE != kLayerNorm) v += cur.ok1 ? (float)cur.b[j].v[e] : 0.0f;
+        if (MODE == kEmb) v += cur.ok2 ? (float)cur.c[j].v[e] : 0.0f;
+        x[j][e] = MODE == kEmb ? v : v + bi[j][e];
       }
-#pragma unroll
-      for (int j = 0; j < NV; ++j)
-#pragma unroll
-        for (int e = 0; e < VEC; ++e)
-          x[j][e] = (wok ? (float)a[j].v[e] : 0.0f) + (pok ? (float)p[j].v[e] : 0.0f) +
-                    (gok ? (float)q[j].v[e] : 0.0f);
-    } else {
-      const T* ip = static_cast<const T*>(L.input) + r * L.ld;
-      const T* sp = static_cast<const T*>(L.skip) + r * L.ld;
-      Pack<T, VEC> a[NV], k[NV];
-#pragma unroll
-      for (int j = 0; j < NV; ++j) {
-        const int cc = live[j] ? (j * 64 + lane) * VEC : 0;
-        a[j] = *reinterpret_cast<const Pack<T, VEC>*>(ip + cc);
-        if (MODE == kSkip) k[j] = *reinterpret_cast<const Pack<T, VEC>*>(sp + cc);
-      }
-#pragma unroll
-      for (int j = 0; j < NV; ++j)
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          float v = (float)a[j].v[e];
-          if (MODE == kSkip) v += (float)k[j].v[e];
-          x[j][e] = v + bi[j][e];
-        }
-    }
 
     // lane-local statistics, then the wave-wide merge
     float sum = 0.0f;
@@ -212,16 +234,17 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
     const float mu = w.mean;
     const float rs = 1.0f / sqrtf(w.m2 / w.n + L.eps);
 
-    T* op = static_cast<T*>(L.output) + r * L.ld;
+    T FWDMI_GLOBAL* op = gmut<T>(L.output) + r * L.ld;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       if (live[j]) {
         Pack<T, VEC> o;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o.v[e] = (T)(g[j][e] * ((x[j][e] - mu) * rs) + be[j][e]);
-        *reinterpret_cast<Pack<T, VEC>*>(op + (j * 64 + lane) * VEC) = o;
+        gstore<T, VEC>(op + col[j], o);
       }
     }
+    cur = nxt;
   }
   if (oob && L.oob_flag) atomicOr(L.oob_flag, 1);
 }
@@ -298,7 +321,7 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
   }();
   // Enough wavefronts to fill the chip; beyond that a wavefront loops over rows so the
   // gamma/beta registers are reused.
-  const int64_t max_blocks = (int64_t)cus * 8;
+  const int64_t max_blocks = (int64_t)cus * FWDMI_LN_BLOCKS_PER_CU;
   const int64_t want = (L.rows + kWavesPerWG - 1) / kWavesPerWG;
   L.row_blocks = (int)std::max<int64_t>(1, std::min(want, max_blocks));
   L.total_waves = L.row_blocks * kWavesPerWG;

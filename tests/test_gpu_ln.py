@@ -167,3 +167,38 @@ def test_plugins_config5_chain(oracle):
     # a half-precision plugin refuses float input at configure time
     with pytest.raises(lib.FwdmiError):
         skip.configurePlugin([((64, 4, 1024), lib.F32)] * 2, [((64, 4, 1024), lib.F32)])
+
+
+def test_launches_can_be_captured_in_a_hip_graph(oracle):
+    """enqueue allocates nothing and never synchronises, so a chain of launches can be captured
+    once and replayed; every replay (with eager work in between) must equal the eager result."""
+    wl = workloads.config5(variant=2, batch=4, seq=64)
+    a = [dev(wl.input_ids), dev(wl.segment_ids), dev(wl.input_mask), dev(wl.word), dev(wl.pos), dev(wl.tok),
+         f32(wl.gamma), f32(wl.beta)]
+    sk, g, b, bi = dev(wl.skip), f32(wl.skip_gamma), f32(wl.skip_beta), f32(wl.skip_bias)
+    emb = torch.empty((64, 4, 1024), dtype=torch.float16, device="cuda")
+    midx = torch.empty((4,), dtype=torch.int32, device="cuda")
+    out = torch.empty_like(emb)
+    bw = workloads.config2(variant=6, table_dtype=np.float16, rows=5000, n_bags=300)
+    tb, ix, of = dev(bw.table), dev(bw.indices), dev(bw.offsets)
+    bag_out = torch.empty((300, 128), dtype=torch.float16, device="cuda")
+
+    def chain():
+        ops.emb_layer_norm(*a, eps=wl.eps, out=emb, mask_idx=midx)
+        ops.skip_layer_norm(emb, g, b, skip=sk, bias=bi, eps=wl.eps, out=out)
+        ops.embedding_bag(tb, ix, of, "sum", out=bag_out)
+
+    chain()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (emb, midx, out, bag_out)]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        chain()
+    for i in range(4):
+        for t in (emb, midx, out, bag_out):
+            t.fill_(0)                                   # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, w in zip((emb, midx, out, bag_out), want):
+            assert torch.equal(got, w), "replay %d differs from the eager result" % i

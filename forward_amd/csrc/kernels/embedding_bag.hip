@@ -167,8 +167,14 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
 
   const TW FWDMI_GLOBAL* __restrict__ tab = gconst<TW>(T.data);
   const int n_units = nb * L.n_slices;
-  // 32-bit id arithmetic is exact when ids are int32 and the table's id range lies in [0, 2^31).
-  const bool narrow = sizeof(TI) == 4 && T.data_offset >= 0 && T.data_offset + T.count <= ((int64_t)1 << 31);
+  // Conditions of the 32-bit ("compact") id / address arithmetic, uniform over the workgroup.
+  const uint32_t row_bytes = (uint32_t)L.dim * (uint32_t)sizeof(TW);
+  const bool compact = sizeof(TI) == 4 && T.data_offset >= 0 && T.data_offset + T.count <= ((int64_t)1 << 31) &&
+                       T.count <= (1 << 24) && row_bytes < (1u << 24) &&
+                       (uint64_t)T.count * row_bytes <= ((uint64_t)1 << 32);
+  const uint32_t lo32 = (uint32_t)T.data_offset;
+  const uint32_t last32 = (uint32_t)(T.count - 1);
+  const char FWDMI_GLOBAL* const tab_bytes = gconst<char>(T.data);
   bool oob = false;
   const float one = L.one;
 
@@ -182,6 +188,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     const int col = (sl * G + gl) * VEC;
     const bool col_ok = col < L.dim;
     const TW FWDMI_GLOBAL* __restrict__ tcol = tab + (col_ok ? col : 0);
+    const uint32_t col_bytes = (uint32_t)(col_ok ? col : 0) * (uint32_t)sizeof(TW);
     // A run whose offsets decrease can make [start,end) leave the staged window.
     const bool in_lds = staged && start >= span0 && end <= span0 + span;
 
@@ -194,52 +201,70 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     bool first = true;
 
     // Loads UU rows starting at bag position i (all loads issued before the first use), then
-    // folds them in bag order.  LDS selects where the ids come from; NARROW selects 32-bit id
-    // arithmetic (valid when every in-range id is a non-negative int32).
-    auto step = [&](auto uu_tag, auto lds_tag, auto narrow_tag, int64_t i) {
+    // folds them in bag order.  LDS selects where the ids come from.  COMPACT selects 32-bit
+    // arithmetic: ids are int32, every in-range id is non-negative, the table has at most 2^24
+    // rows and 4 GiB, so a row's byte offset is one 24-bit multiply-add on top of a uniform base.
+    auto step = [&](auto uu_tag, auto lds_tag, auto compact_tag, int64_t i) {
       constexpr int UU = decltype(uu_tag)::value;
       constexpr bool LDS = decltype(lds_tag)::value;
-      constexpr bool NARROW = decltype(narrow_tag)::value;
+      constexpr bool COMPACT = decltype(compact_tag)::value;
       Pack<TW, VEC> v[UU];
       TI id[UU];
       float w[UU];
       bool ok[UU];
       bool all_ok = true;
+      if (LDS) {
+        // one LDS address per step; the unrolled reads use immediate offsets
+        const uint32_t li = (uint32_t)(i - span0);
+        const TI* const sp = s_idx + li;
+        const float* const wp = s_w + li;
 #pragma unroll
-      for (int u = 0; u < UU; ++u) {
-        const int64_t p = i + u;
-        if (LDS) {
-          id[u] = s_idx[(int)(p - span0)];
-          if (KIND == kWeighted) w[u] = s_w[(int)(p - span0)];
-        } else {
-          id[u] = ids[p];
-          if (KIND == kWeighted) w[u] = (float)psw[p];
+        for (int u = 0; u < UU; ++u) {
+          id[u] = sp[u];
+          if (KIND == kWeighted) w[u] = wp[u];
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+          id[u] = ids[i + u];
+          if (KIND == kWeighted) w[u] = (float)psw[i + u];
         }
       }
+      // a bad id never forms an address: a valid row is fetched instead and discarded below
+      if (COMPACT) {
+        uint32_t worst = 0;
 #pragma unroll
-      for (int u = 0; u < UU; ++u) {
-        // a bad id never forms an address: row 0 is fetched instead and discarded below
-        if (NARROW) {
-          const uint32_t row = (uint32_t)id[u] - (uint32_t)T.data_offset;
-          ok[u] = row < (uint32_t)T.count;
-          v[u] = gload<TW, VEC>(tcol + (uint64_t)(ok[u] ? row : 0u) * (uint32_t)L.dim);
-        } else {
+        for (int u = 0; u < UU; ++u) {
+          const uint32_t row = (uint32_t)id[u] - lo32;
+          worst = max(worst, row);
+          const uint32_t off = __umul24(min(row, last32), row_bytes) + col_bytes;
+          v[u] = gload<TW, VEC>(reinterpret_cast<const TW FWDMI_GLOBAL*>(tab_bytes + off));
+          if (KIND == kMax) ok[u] = row <= last32;
+        }
+        all_ok = worst <= last32;
+      } else {
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
           const uint64_t row = (uint64_t)((int64_t)id[u] - T.data_offset);
           ok[u] = row < (uint64_t)T.count;
           v[u] = gload<TW, VEC>(tcol + (ok[u] ? row : 0) * (uint64_t)L.dim);
+          all_ok &= ok[u];
         }
-        all_ok &= ok[u];
       }
       if (__builtin_expect(!__all(all_ok), 0)) {
         oob |= !all_ok;
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
+          if (COMPACT) ok[u] = ((uint32_t)id[u] - lo32) <= last32;
           if (!ok[u]) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) v[u].v[e] = (TW)0.0f;
             w[u] = 0.0f;
           }
         }
+      } else if (COMPACT && KIND != kMax) {
+#pragma unroll
+        for (int u = 0; u < UU; ++u) ok[u] = true;
       }
 #pragma unroll
       for (int u = 0; u < UU; ++u) {
@@ -265,21 +290,21 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
         if (KIND == kMax && ok[u]) first = false;
       }
     };
-    auto bag = [&](auto lds_tag, auto narrow_tag) {
+    auto bag = [&](auto lds_tag, auto compact_tag) {
       int64_t i = start;
-      for (; i + kUnroll <= end; i += kUnroll) step(std::integral_constant<int, kUnroll>{}, lds_tag, narrow_tag, i);
+      for (; i + kUnroll <= end; i += kUnroll) step(std::integral_constant<int, kUnroll>{}, lds_tag, compact_tag, i);
       if (i + 4 <= end) {
-        step(std::integral_constant<int, 4>{}, lds_tag, narrow_tag, i);
+        step(std::integral_constant<int, 4>{}, lds_tag, compact_tag, i);
         i += 4;
       }
       if (i + 2 <= end) {
-        step(std::integral_constant<int, 2>{}, lds_tag, narrow_tag, i);
+        step(std::integral_constant<int, 2>{}, lds_tag, compact_tag, i);
         i += 2;
       }
-      if (i < end) step(std::integral_constant<int, 1>{}, lds_tag, narrow_tag, i);
+      if (i < end) step(std::integral_constant<int, 1>{}, lds_tag, compact_tag, i);
     };
     if (in_lds) {
-      if (narrow)
+      if (compact)
         bag(std::true_type{}, std::true_type{});
       else
         bag(std::true_type{}, std::false_type{});

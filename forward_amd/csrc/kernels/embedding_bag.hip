@@ -35,6 +35,7 @@ constexpr int kWG = 256;           // lanes per workgroup (large batches; small 
 constexpr int kIdxBytes = 16384;   // LDS bytes for staged ids per workgroup (4096 int32 / 2048 int64)
 constexpr int kXcds = 8;           // accelerator complex dies; workgroup b is dispatched to XCD b % 8
 constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
+constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting sort
 #ifndef FWDMI_BAG_UNROLL
 #define FWDMI_BAG_UNROLL 8
 #endif
@@ -82,6 +83,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   int* const s_len = reinterpret_cast<int*>(s_w + (KIND == kWeighted ? L.idx_cap : 0));
   uint16_t* const s_order = reinterpret_cast<uint16_t*>(s_len + L.bags_per_wg);
   __shared__ int s_next;
+  __shared__ int s_hist[kLenBuckets];
   const int kIdxCap = L.idx_cap;
   const int wg_lanes = blockDim.x;
 
@@ -132,6 +134,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     s_off[i] = min(max(v, (int64_t)0), T.input_size);
   }
   if (tid == 0) s_next = slots;
+  for (int i = tid; i < kLenBuckets; i += wg_lanes) s_hist[i] = 0;
   __syncthreads();
 
   // ---- stage the ids (and weights) the run covers ----------------------------------------
@@ -151,16 +154,39 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   // The order changes which slot reduces a bag, never the result.
   const bool sorted = L.fixed_len < 0 && nb > 1;
   if (sorted) {
-    for (int i = tid; i < nb; i += wg_lanes) s_len[i] = (int)min(max(s_off[i + 1] - s_off[i], (int64_t)0), (int64_t)INT_MAX);
+    // Counting sort on min(length, 255), descending: histogram with LDS atomics, exclusive scan
+    // of the 256 buckets by the first wavefront, scatter.  (Order inside a bucket is arbitrary.)
+    for (int i = tid; i < nb; i += wg_lanes) {
+      const int len = (int)min(max(s_off[i + 1] - s_off[i], (int64_t)0), (int64_t)(kLenBuckets - 1));
+      const int bucket = kLenBuckets - 1 - len;
+      s_len[i] = (bucket << 16) | atomicAdd(&s_hist[bucket], 1);
+    }
+    __syncthreads();
+    if (tid < 64) {
+      constexpr int kPer = kLenBuckets / 64;
+      int c[kPer], sum = 0;
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        c[j] = s_hist[tid * kPer + j];
+        sum += c[j];
+      }
+      int incl = sum;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (tid >= d) incl += up;
+      }
+      int run = incl - sum;
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        s_hist[tid * kPer + j] = run;
+        run += c[j];
+      }
+    }
     __syncthreads();
     for (int i = tid; i < nb; i += wg_lanes) {
-      const int li = s_len[i];
-      int rank = 0;
-      for (int j = 0; j < nb; ++j) {
-        const int lj = s_len[j];
-        rank += (lj > li || (lj == li && j < i)) ? 1 : 0;
-      }
-      s_order[rank] = (uint16_t)i;
+      const int packed = s_len[i];
+      s_order[s_hist[packed >> 16] + (packed & 0xffff)] = (uint16_t)i;
     }
   }
   __syncthreads();

@@ -32,18 +32,22 @@ namespace fwdmi {
 namespace {
 
 constexpr int kWG = 256;           // lanes per workgroup (large batches; small ones use 128 or 64)
-constexpr int kIdxBytes = 16384;   // LDS bytes for staged ids per workgroup (4096 int32 / 2048 int64)
+#ifndef FWDMI_BAG_IDX_BYTES
+#define FWDMI_BAG_IDX_BYTES 16384
+#endif
+constexpr int kIdxBytes = FWDMI_BAG_IDX_BYTES;   // LDS bytes for staged ids per workgroup (4096 int32 / 2048 int64)
 constexpr int kXcds = 8;           // accelerator complex dies; workgroup b is dispatched to XCD b % 8
 constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
 constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting sort
 #ifndef FWDMI_BAG_UNROLL
 #define FWDMI_BAG_UNROLL 8
 #endif
-#ifdef FWDMI_BAG_WAVES_PER_EU
-#define FWDMI_BAG_OCCUPANCY __attribute__((amdgpu_waves_per_eu(FWDMI_BAG_WAVES_PER_EU)))
-#else
-#define FWDMI_BAG_OCCUPANCY
+#ifndef FWDMI_BAG_WAVES_PER_EU
+#define FWDMI_BAG_WAVES_PER_EU 6  // register budget of 80 VGPRs: measured best on the 26-table configuration
 #endif
+// max mode, weights and 64-bit ids carry more live registers: they keep the looser budget
+#define FWDMI_BAG_OCCUPANCY \
+  __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kWeighted || sizeof(TI) == 8) ? 4 : FWDMI_BAG_WAVES_PER_EU)))
 constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 
 enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3 };

@@ -29,7 +29,7 @@ def log(*a):
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="config4", choices=["config4"])
     ap.add_argument("--tables", type=int, default=26, help="debug only: fewer tables (not the named config)")
@@ -146,7 +146,45 @@ def cpu_baseline(wl, tabs_dev, n_cpu_bags, torch):
     return res, out, nb
 
 
-def extra_measurements(torch, ops, workloads, steps):
+def copy_bandwidth(torch):
+    """Device-to-device copy of 1 GiB (read + write), GB/s: what a streaming kernel gets on this box."""
+    src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+    dst = torch.empty_like(src)
+    _, per = time_events(torch, lambda: dst.copy_(src), 10, 3)
+    return 2 * src.numel() * 4 / (float(np.median(per)) * 1e-3) / 1e9
+
+
+def cpu_bert(torch, wl, threads):
+    """libtorch CPU tokens/s of embedding x3 + add + layer_norm (+ residual/bias add + layer_norm)."""
+    tw, tp, tt = (torch.from_numpy(a) for a in (wl.word, wl.pos, wl.tok))
+    ids, seg = torch.from_numpy(wl.input_ids).long(), torch.from_numpy(wl.segment_ids).long()
+    g, b = torch.from_numpy(wl.gamma), torch.from_numpy(wl.beta)
+    S, H = wl.input_ids.shape[0], wl.word.shape[1]
+    F = torch.nn.functional
+    sk = None if wl.skip is None else [torch.from_numpy(a) for a in (wl.skip, wl.skip_bias, wl.skip_gamma, wl.skip_beta)]
+
+    def run():
+        e = F.layer_norm(F.embedding(ids, tw) + tp[:S].unsqueeze(1) + F.embedding(seg, tt), (H,), g, b, wl.eps)
+        if sk is not None:
+            e = F.layer_norm(e + sk[0] + sk[1], (H,), sk[2], sk[3], wl.eps)
+        return e
+
+    res = {}
+    for n in threads:
+        torch.set_num_threads(n)
+        for _ in range(3):
+            run()
+        ts = []
+        for _ in range(10):
+            t0 = time.perf_counter()
+            run()
+            ts.append(time.perf_counter() - t0)
+        res["threads_%d" % n] = wl.n_tokens / float(np.median(ts))
+    torch.set_num_threads(threads[0])
+    return res
+
+
+def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
     """Tokens/s of the BERT configs and bags/s of config 2.  These launches take ~10 us, less than
     a Python launch costs, so they are timed as HIP-graph replays (GPU time, launch gaps included)."""
     ex = {}
@@ -162,6 +200,9 @@ def extra_measurements(torch, ops, workloads, steps):
         ms = time_graph(torch, fn)
         ex[name] = {"tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
                     "algorithmic_GBs": wl.emb_algorithmic_bytes() / (ms * 1e-3) / 1e9}
+        if with_cpu:
+            cores = min(16, os.cpu_count() or 1)
+            ex[name.split("_")[0] + "_libtorch_cpu_tokens_per_s"] = cpu_bert(torch, wl, (cores, 1))
         if wl.skip is not None:
             x, sk = out, dev(wl.skip)
             g, b, bi = f32(wl.skip_gamma), f32(wl.skip_beta), f32(wl.skip_bias)
@@ -170,6 +211,14 @@ def extra_measurements(torch, ops, workloads, steps):
             ms = time_graph(torch, fn2)
             ex["config5_skip_layer_norm"] = {"tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
                                              "algorithmic_GBs": wl.skip_algorithmic_bytes() / (ms * 1e-3) / 1e9}
+            # the same two stages in one pass (no intermediate round trip through HBM)
+            fn3 = lambda: ops.emb_layer_norm(*a, eps=wl.eps, out=o2, mask_idx=midx, skip=sk, gamma2=g, beta2=b,
+                                             bias2=bi, eps2=wl.eps)
+            ms = time_graph(torch, fn3)
+            h2 = wl.n_tokens * wl.word.shape[1] * wl.word.itemsize
+            ex["config5_fused_emb_skip_layer_norm"] = {
+                "tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
+                "algorithmic_GBs": (wl.emb_algorithmic_bytes() + wl.skip_algorithmic_bytes() - 2 * h2) / (ms * 1e-3) / 1e9}
     for tdt, tname in ((np.float32, "fp32"), (np.float16, "fp16")):
         wl = workloads.config2(table_dtype=tdt)
         tb, ix, of = dev(wl.table), dev(wl.indices), dev(wl.offsets)
@@ -226,11 +275,12 @@ def main():
         "metric": "EmbeddingBag bags/sec + achieved HBM GB/s (% peak), 26-table fp16 batch 64K",
         "value": total_bags / (ms_per_step * 1e-3), "unit": "bags/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 rows, f32 accumulate", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config4: DLRM sparse stage, %d tables x %d bags, dim %d fp16, int32 ids, "
                                "Zipf(1.1) ids and bag lengths (mean %.2f), fp16 output [%d, %d]%s"
                                % (len(wl.rows), wl.n_bags, wl.dim, wl.n_indices() / total_bags, wl.n_bags,
                                   batch.width, "" if (args.tables == 26 and args.bags == 65536) else " (REDUCED, debug)"),
+                   "storage": "fp16 rows and output, fp32 accumulation, int32 ids",
                    "launch": "per-table" if args.per_table else "fused multi-table",
                    "total_ids": wl.n_indices(), "table_bytes": int(sum(t.numel() * 2 for t in tabs))},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -261,7 +311,8 @@ def main():
         log("cpu baseline leg %.1fs" % (time.time() - t1))
     if not args.no_extra:
         del tabs, batch
-        result["extra"] = extra_measurements(torch, ops, workloads, max(10, args.steps))
+        result["extra"] = extra_measurements(torch, ops, workloads, max(10, args.steps), with_cpu=not args.no_cpu)
+        result["extra"]["device_copy_GBs"] = copy_bandwidth(torch)
     print(json.dumps(result), flush=True)
 
 

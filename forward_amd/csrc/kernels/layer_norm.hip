@@ -16,6 +16,10 @@
 #include "../common.h"
 #include "device_util.h"
 
+// No implicit multiply-add fusion in this file: the fused kernel and the separate launches must
+// round identically, so every fused operation is written as an explicit fma.
+#pragma clang fp contract(off)
+
 namespace fwdmi {
 namespace {
 
@@ -25,7 +29,8 @@ namespace {
 constexpr int kWG = 256;
 constexpr int kWavesPerWG = kWG / 64;
 
-enum Mode { kLayerNorm = 0, kSkip = 1, kEmb = 2 };
+enum Mode { kLayerNorm = 0, kSkip = 1, kEmb = 2, kEmbSkip = 3 };
+constexpr bool is_emb(int mode) { return mode == kEmb || mode == kEmbSkip; }
 
 struct LnLaunch {
   const void* input;  // kLayerNorm / kSkip: [rows, ld]; kEmb: word table
@@ -35,6 +40,10 @@ struct LnLaunch {
   const float* gamma;
   const float* beta;
   const float* bias;  // nullable
+  const float* gamma2;  // kEmbSkip: parameters of the second LayerNorm
+  const float* beta2;
+  const float* bias2;   // nullable
+  void* emb_output;     // kEmbSkip: optional copy of the first-stage result
   void* output;
   const int32_t* input_ids;
   const int32_t* segment_ids;
@@ -48,7 +57,19 @@ struct LnLaunch {
   int32_t row_blocks;  // workgroups that process rows; the rest compute mask indices
   int32_t total_waves; // row-processing wavefronts in the grid
   float eps;
+  float eps2;
+  int32_t batch_major;  // kEmb*: ids / mask are [B,S] and rows are ordered b*S + s
 };
+
+// Rounds an fp32 result to the I/O type in a step of its own.  Without the barrier the compiler
+// may fold the preceding fma and the conversion into one mixed-precision instruction that rounds
+// once; whether it does depends on the surrounding code, and the fused and the two-launch forms
+// of the same arithmetic would then differ in the last bit.
+template <typename T>
+__device__ __forceinline__ T round_to(float y) {
+  asm volatile("" : "+v"(y));
+  return (T)y;
+}
 
 struct Welford {
   float n, mean, m2;
@@ -99,11 +120,13 @@ __device__ __forceinline__ int wave_min(int v) {
   return v;
 }
 
-// Index of the first zero of mask column b ([S,B] layout), S when there is none.
+// Index of the first zero of the mask of batch row b, S when there is none.
 __device__ __forceinline__ void mask_index_wave(const LnLaunch& L, int b, int lane) {
   int first = L.S;
+  const int64_t base = L.batch_major ? (int64_t)b * L.S : b;
+  const int64_t step = L.batch_major ? 1 : L.B;
   for (int s = lane; s < L.S; s += 64)
-    if (L.input_mask[(int64_t)s * L.B + b] == 0) {
+    if (L.input_mask[base + (int64_t)s * step] == 0) {
       first = s;
       break;
     }
@@ -116,7 +139,8 @@ template <typename T, int VEC, int NV, int MODE>
 struct RowRegs {
   Pack<T, VEC> a[NV];                        // input / word row
   Pack<T, VEC> b[MODE == kLayerNorm ? 1 : NV];  // skip / position row
-  Pack<T, VEC> c[MODE == kEmb ? NV : 1];     // token-type row
+  Pack<T, VEC> c[is_emb(MODE) ? NV : 1];     // token-type row
+  Pack<T, VEC> d[MODE == kEmbSkip ? NV : 1]; // residual of the fused second stage
   bool ok0, ok1, ok2;
 };
 
@@ -125,7 +149,7 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   const int lane = threadIdx.x & 63;
   const int wave_in_wg = threadIdx.x >> 6;
   if ((int)blockIdx.x >= L.row_blocks) {
-    if (MODE == kEmb) {
+    if (is_emb(MODE)) {
       const int b = ((int)blockIdx.x - L.row_blocks) * kWavesPerWG + wave_in_wg;
       if (b < L.B) mask_index_wave(L, b, lane);
     }
@@ -133,7 +157,8 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   }
   const int wave = blockIdx.x * kWavesPerWG + wave_in_wg;
   const T FWDMI_GLOBAL* const in0 = gconst<T>(L.input);
-  const T FWDMI_GLOBAL* const in1 = gconst<T>(MODE == kEmb ? L.pos : L.skip);
+  const T FWDMI_GLOBAL* const in1 = gconst<T>(is_emb(MODE) ? L.pos : L.skip);
+  const T FWDMI_GLOBAL* const in3 = gconst<T>(L.skip);
   const T FWDMI_GLOBAL* const in2 = gconst<T>(L.tok);
   const int32_t FWDMI_GLOBAL* const ids = gconst<int32_t>(L.input_ids);
   const int32_t FWDMI_GLOBAL* const segs = gconst<int32_t>(L.segment_ids);
@@ -154,8 +179,8 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   using Regs = RowRegs<T, VEC, NV, MODE>;
   // Issues the loads of row r (no use of the data yet).
   auto fetch = [&](int64_t r, Regs& R) {
-    if (MODE == kEmb) {
-      const int s = (int)(r / L.B);
+    if (is_emb(MODE)) {
+      const int s = L.batch_major ? (int)(r % L.S) : (int)(r / L.B);
       const int64_t w = ids[r], sg = segs[r];
       R.ok0 = w >= 0 && w < L.word_count;
       R.ok1 = s < L.pos_count;
@@ -168,6 +193,7 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
         R.a[j] = gload<T, VEC>(wp + col[j]);
         R.b[j] = gload<T, VEC>(pp + col[j]);
         R.c[j] = gload<T, VEC>(tp + col[j]);
+        if (MODE == kEmbSkip) R.d[j] = gload<T, VEC>(in3 + r * L.ld + col[j]);
       }
     } else {
       R.ok0 = R.ok1 = R.ok2 = true;
@@ -205,43 +231,78 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
     if (rn < L.rows) fetch(rn, nxt);
 
     float x[NV][VEC];
-    if (MODE == kEmb) oob |= !(cur.ok0 && cur.ok1 && cur.ok2);
+    if (is_emb(MODE)) oob |= !(cur.ok0 && cur.ok1 && cur.ok2);
 #pragma unroll
     for (int j = 0; j < NV; ++j)
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
         float v = cur.ok0 ? (float)cur.a[j].v[e] : 0.0f;
         if (MODE != kLayerNorm) v += cur.ok1 ? (float)cur.b[j].v[e] : 0.0f;
-        if (MODE == kEmb) v += cur.ok2 ? (float)cur.c[j].v[e] : 0.0f;
-        x[j][e] = MODE == kEmb ? v : v + bi[j][e];
+        if (is_emb(MODE)) v += cur.ok2 ? (float)cur.c[j].v[e] : 0.0f;
+        x[j][e] = is_emb(MODE) ? v : v + bi[j][e];
       }
 
-    // lane-local statistics, then the wave-wide merge
-    float sum = 0.0f;
+    // lane-local statistics, then the wave-wide merge: returns (mean, 1/sigma)
+    auto stats = [&](float eps, float& mu, float& rs) {
+      float sum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < NV; ++j)
+      for (int j = 0; j < NV; ++j)
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) sum += live[j] ? x[j][e] : 0.0f;
-    Welford w{cnt, sum * inv_cnt, 0.0f};
+        for (int e = 0; e < VEC; ++e) sum += live[j] ? x[j][e] : 0.0f;
+      Welford w{cnt, sum * inv_cnt, 0.0f};
 #pragma unroll
-    for (int j = 0; j < NV; ++j)
+      for (int j = 0; j < NV; ++j)
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float d = live[j] ? x[j][e] - w.mean : 0.0f;
-        w.m2 = __builtin_fmaf(d, d, w.m2);
-      }
-    w = wave_allreduce(w);
-    const float mu = w.mean;
-    const float rs = 1.0f / sqrtf(w.m2 / w.n + L.eps);
+        for (int e = 0; e < VEC; ++e) {
+          const float d = live[j] ? x[j][e] - w.mean : 0.0f;
+          w.m2 = __builtin_fmaf(d, d, w.m2);
+        }
+      w = wave_allreduce(w);
+      mu = w.mean;
+      rs = 1.0f / sqrtf(w.m2 / w.n + eps);
+    };
+    float mu, rs;
+    stats(L.eps, mu, rs);
 
-    T FWDMI_GLOBAL* op = gmut<T>(L.output) + r * L.ld;
+    if (MODE != kEmbSkip) {
+      T FWDMI_GLOBAL* op = gmut<T>(L.output) + r * L.ld;
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      if (live[j]) {
+      for (int j = 0; j < NV; ++j) {
+        if (live[j]) {
+          Pack<T, VEC> o;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) o.v[e] = round_to<T>(__builtin_fmaf(g[j][e], (x[j][e] - mu) * rs, be[j][e]));
+          gstore<T, VEC>(op + col[j], o);
+        }
+      }
+    } else {
+      // Fused second stage: the first result is rounded to the I/O type exactly as if it had
+      // been stored and read back, then out = LN2(first + residual (+ bias2)).
+      T FWDMI_GLOBAL* ep = L.emb_output ? gmut<T>(L.emb_output) + r * L.ld : nullptr;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
         Pack<T, VEC> o;
+        Pack<float, VEC> b2{};
+        if (L.bias2) b2 = gload<float, VEC>(gconst<float>(L.bias2) + col[j]);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) o.v[e] = (T)(g[j][e] * ((x[j][e] - mu) * rs) + be[j][e]);
-        gstore<T, VEC>(op + col[j], o);
+        for (int e = 0; e < VEC; ++e) {
+          o.v[e] = round_to<T>(__builtin_fmaf(g[j][e], (x[j][e] - mu) * rs, be[j][e]));
+          x[j][e] = (float)o.v[e] + (float)cur.d[j].v[e] + (L.bias2 ? b2.v[e] : 0.0f);
+        }
+        if (ep && live[j]) gstore<T, VEC>(ep + col[j], o);
+      }
+      stats(L.eps2, mu, rs);
+      T FWDMI_GLOBAL* op = gmut<T>(L.output) + r * L.ld;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        if (live[j]) {
+          const Pack<float, VEC> g2 = gload<float, VEC>(gconst<float>(L.gamma2) + col[j]);
+          const Pack<float, VEC> be2 = gload<float, VEC>(gconst<float>(L.beta2) + col[j]);
+          Pack<T, VEC> o;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) o.v[e] = round_to<T>(__builtin_fmaf(g2.v[e], (x[j][e] - mu) * rs, be2.v[e]));
+          gstore<T, VEC>(op + col[j], o);
+        }
       }
     }
     cur = nxt;
@@ -267,7 +328,7 @@ __global__ __launch_bounds__(kWG) void ln_strided_kernel(const LnLaunch L) {
     const T *p0 = nullptr, *p1 = nullptr, *p2 = nullptr;
     bool ok0 = true, ok1 = false, ok2 = false;
     if (MODE == kEmb) {
-      const int s = (int)(r / L.B);
+      const int s = L.batch_major ? (int)(r % L.S) : (int)(r / L.B);
       const int64_t w = L.input_ids[r], sg = L.segment_ids[r];
       ok0 = w >= 0 && w < L.word_count;
       ok1 = s < L.pos_count;
@@ -302,7 +363,7 @@ __global__ __launch_bounds__(kWG) void ln_strided_kernel(const LnLaunch L) {
     const float mu = w.mean;
     const float rs = 1.0f / sqrtf(w.m2 / w.n + L.eps);
     T* op = static_cast<T*>(L.output) + r * L.ld;
-    for (int i = lane; i < L.ld; i += 64) op[i] = (T)(L.gamma[i] * ((fetch(i) - mu) * rs) + L.beta[i]);
+    for (int i = lane; i < L.ld; i += 64) op[i] = round_to<T>(__builtin_fmaf(L.gamma[i], (fetch(i) - mu) * rs, L.beta[i]));
   }
   if (oob && L.oob_flag) atomicOr(L.oob_flag, 1);
 }
@@ -325,7 +386,7 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
   const int64_t want = (L.rows + kWavesPerWG - 1) / kWavesPerWG;
   L.row_blocks = (int)std::max<int64_t>(1, std::min(want, max_blocks));
   L.total_waves = L.row_blocks * kWavesPerWG;
-  const int mask_blocks = (MODE == kEmb && L.mask_idx) ? (L.B + kWavesPerWG - 1) / kWavesPerWG : 0;
+  const int mask_blocks = (is_emb(MODE) && L.mask_idx) ? (L.B + kWavesPerWG - 1) / kWavesPerWG : 0;
   const dim3 grid(L.row_blocks + mask_blocks), block(kWG);
 
   const int chunks = (L.ld + 64 * kVec - 1) / (64 * kVec);
@@ -338,11 +399,19 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
       hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 4, MODE>), grid, block, 0, stream, L);
     else
       hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 8, MODE>), grid, block, 0, stream, L);
+  } else if constexpr (MODE == kEmbSkip) {
+    return set_error(FWDMI_ERR_UNSUPPORTED, "fused emb+skip layer norm needs 16-byte sliceable rows");
   } else {
     hipLaunchKernelGGL((ln_strided_kernel<T, MODE>), grid, block, 0, stream, L);
   }
   FWDMI_HIP_CHECK(hipGetLastError());
   return FWDMI_OK;
+}
+
+// True when rows of `ld` elements of `dtype` can take the register-resident kernel.
+bool rows_kernel_ok(int ld, int dtype, bool vec_ok) {
+  const int vec = 16 / (int)dtype_size(dtype);
+  return vec_ok && ld % vec == 0 && (ld + 64 * vec - 1) / (64 * vec) <= 8;
 }
 
 template <int MODE>
@@ -388,11 +457,12 @@ int fwdmi_layer_norm(void* stream, int32_t ld, int64_t n, const void* input, con
   return fwdmi_skip_layer_norm(stream, ld, n, input, nullptr, beta, gamma, output, bias, dtype, eps);
 }
 
-int fwdmi_emb_layer_norm(void* stream, int32_t S, int32_t B, int32_t ld, const int32_t* input_ids,
-                         const int32_t* segment_ids, const int32_t* input_mask, const float* beta,
-                         const float* gamma, const void* word, const void* pos, const void* tok,
-                         int32_t word_count, int32_t pos_count, int32_t tok_count, void* output,
-                         int32_t* mask_idx, int32_t dtype, float eps, int32_t* oob_flag) {
+int fwdmi_emb_layer_norm_ex(void* stream, int32_t S, int32_t B, int32_t ld, const int32_t* input_ids,
+                            const int32_t* segment_ids, const int32_t* input_mask, const float* beta,
+                            const float* gamma, const void* word, const void* pos, const void* tok,
+                            int32_t word_count, int32_t pos_count, int32_t tok_count, void* output,
+                            int32_t* mask_idx, int32_t dtype, float eps, int32_t* oob_flag,
+                            const fwdmi_emb_ext* ext) {
   using namespace fwdmi;
   clear_error();
   if (!is_float_dtype(dtype)) return set_error(FWDMI_ERR_UNSUPPORTED, "emb layer norm: unsupported dtype %d", dtype);
@@ -402,6 +472,8 @@ int fwdmi_emb_layer_norm(void* stream, int32_t S, int32_t B, int32_t ld, const i
                 "emb layer norm: null pointer");
   FWDMI_REQUIRE(word_count > 0 && pos_count > 0 && tok_count > 0, "emb layer norm: empty table");
   FWDMI_REQUIRE(!mask_idx || input_mask, "emb layer norm: mask_idx requested without input_mask");
+  const bool fused = ext && ext->skip;
+  FWDMI_REQUIRE(!fused || (ext->gamma2 && ext->beta2), "emb layer norm: fused stage needs gamma2 and beta2");
   LnLaunch L{};
   L.input = word;
   L.pos = pos;
@@ -422,9 +494,39 @@ int fwdmi_emb_layer_norm(void* stream, int32_t S, int32_t B, int32_t ld, const i
   L.pos_count = pos_count;
   L.tok_count = tok_count;
   L.eps = eps;
-  const bool vec_ok = aligned16(word) && aligned16(pos) && aligned16(tok) && aligned16(output) &&
-                      aligned16(gamma) && aligned16(beta);
-  return ln_dispatch<kEmb>(L, dtype, vec_ok, static_cast<hipStream_t>(stream));
+  L.batch_major = ext && ext->batch_major;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  bool vec_ok = aligned16(word) && aligned16(pos) && aligned16(tok) && aligned16(output) && aligned16(gamma) &&
+                aligned16(beta);
+  if (!fused) return ln_dispatch<kEmb>(L, dtype, vec_ok, s);
+
+  vec_ok = vec_ok && aligned16(ext->skip) && aligned16(ext->gamma2) && aligned16(ext->beta2) &&
+           (!ext->bias2 || aligned16(ext->bias2)) && (!ext->emb_output || aligned16(ext->emb_output));
+  if (rows_kernel_ok(ld, dtype, vec_ok)) {
+    L.skip = ext->skip;
+    L.gamma2 = ext->gamma2;
+    L.beta2 = ext->beta2;
+    L.bias2 = ext->bias2;
+    L.eps2 = ext->eps2;
+    L.emb_output = ext->emb_output;
+    return ln_dispatch<kEmbSkip>(L, dtype, vec_ok, s);
+  }
+  // rows that cannot stay in registers: two launches, the second in place over the first result
+  void* first = ext->emb_output ? ext->emb_output : output;
+  L.output = first;
+  int rc = ln_dispatch<kEmb>(L, dtype, false, s);
+  if (rc != FWDMI_OK) return rc;
+  return fwdmi_skip_layer_norm(stream, ld, (int64_t)S * B * ld, first, ext->skip, ext->beta2, ext->gamma2, output,
+                               ext->bias2, dtype, ext->eps2);
+}
+
+int fwdmi_emb_layer_norm(void* stream, int32_t S, int32_t B, int32_t ld, const int32_t* input_ids,
+                         const int32_t* segment_ids, const int32_t* input_mask, const float* beta,
+                         const float* gamma, const void* word, const void* pos, const void* tok,
+                         int32_t word_count, int32_t pos_count, int32_t tok_count, void* output,
+                         int32_t* mask_idx, int32_t dtype, float eps, int32_t* oob_flag) {
+  return fwdmi_emb_layer_norm_ex(stream, S, B, ld, input_ids, segment_ids, input_mask, beta, gamma, word, pos, tok,
+                                 word_count, pos_count, tok_count, output, mask_idx, dtype, eps, oob_flag, nullptr);
 }
 
 }  // extern "C"

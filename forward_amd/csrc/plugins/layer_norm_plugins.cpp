@@ -290,8 +290,9 @@ IPluginV2DynamicExt* LayerNormCreatorBase::deserializePlugin(const char* name, c
 // ================================================================================================
 
 EmbLayerNormPluginDynamic::EmbLayerNormPluginDynamic(std::string name, DataType type, DataType mha_type, int ld,
-                                                     Tables tables, float eps)
-    : layer_name_(std::move(name)), type_(type), mha_type_(mha_type), ld_(ld), eps_(eps), t_(std::move(tables)) {
+                                                     Tables tables, float eps, bool batch_major)
+    : layer_name_(std::move(name)), type_(type), mha_type_(mha_type), ld_(ld), eps_(eps),
+      batch_major_(batch_major), t_(std::move(tables)) {
   std::vector<float> all(t_.beta);
   all.insert(all.end(), t_.gamma.begin(), t_.gamma.end());
   params_ = make_blob_f32(all);
@@ -300,7 +301,7 @@ EmbLayerNormPluginDynamic::EmbLayerNormPluginDynamic(std::string name, DataType 
 EmbLayerNormPluginDynamic::~EmbLayerNormPluginDynamic() noexcept { terminate(); }
 
 IPluginV2DynamicExt* EmbLayerNormPluginDynamic::clone() const noexcept {
-  auto* p = new EmbLayerNormPluginDynamic(layer_name_, type_, mha_type_, ld_, t_, eps_);
+  auto* p = new EmbLayerNormPluginDynamic(layer_name_, type_, mha_type_, ld_, t_, eps_, batch_major_);
   p->params_ = params_;
   p->setPluginNamespace(namespace_.c_str());
   return p;
@@ -308,7 +309,8 @@ IPluginV2DynamicExt* EmbLayerNormPluginDynamic::clone() const noexcept {
 
 // Inputs are three [S, B] id tensors (trt_bert_creator.h:64-71).  Output 0 is the embedding
 // consumed as [S, B, H, 1, 1] (plugins/common/plugin_common.h:39-41); output 1 is the mask index,
-// one int per batch row in the unfused layout (plugin_common.h:63,77-94).
+// one int per batch row in the unfused layout (plugin_common.h:63,77-94).  With the optional
+// `batch_major` field the ids are [B, S] and output 0 is [B, S, H, 1, 1].
 Dims EmbLayerNormPluginDynamic::getOutputDimensions(int outputIndex, const Dims* inputs, int nbInputs) noexcept {
   clear_error();
   if (!inputs || nbInputs != 3 || outputIndex < 0 || outputIndex > 1) {
@@ -323,14 +325,14 @@ Dims EmbLayerNormPluginDynamic::getOutputDimensions(int outputIndex, const Dims*
   Dims out{};
   if (outputIndex == 0) {
     out.nbDims = 5;
-    out.d[0] = inputs[0].d[SDIM];
-    out.d[1] = inputs[0].d[BDIM];
+    out.d[0] = inputs[0].d[0];
+    out.d[1] = inputs[0].d[1];
     out.d[2] = ld_;
     out.d[3] = 1;
     out.d[4] = 1;
   } else {
     out.nbDims = 2;
-    out.d[0] = inputs[0].d[BDIM];
+    out.d[0] = inputs[0].d[batch_major_ ? 0 : BDIM];
     out.d[1] = 1;
   }
   return out;
@@ -390,12 +392,14 @@ int EmbLayerNormPluginDynamic::enqueue(const PluginTensorDesc* inputDesc, const 
   if (inputDesc[0].type != FWDMI_I32 || outputDesc[0].type != (int32_t)type_)
     return set_error(FWDMI_ERR_UNSUPPORTED, "EmbLayerNorm: unsupported types (ids %d, output %d)", inputDesc[0].type,
                      outputDesc[0].type);
-  const int S = inputDesc[0].dims.d[SDIM], B = inputDesc[0].dims.d[BDIM];
-  return fwdmi_emb_layer_norm(hipStream, S, B, ld_, static_cast<const int32_t*>(inputs[0]),
-                              static_cast<const int32_t*>(inputs[1]), static_cast<const int32_t*>(inputs[2]),
-                              d_params_, d_params_ + ld_, d_word_, d_pos_, d_tok_, t_.word_count, t_.pos_count,
-                              t_.tok_count, outputs[0], static_cast<int32_t*>(outputs[1]), (int32_t)type_, eps_,
-                              d_oob_);
+  const int S = inputDesc[0].dims.d[batch_major_ ? 1 : SDIM], B = inputDesc[0].dims.d[batch_major_ ? 0 : BDIM];
+  fwdmi_emb_ext ext{};
+  ext.batch_major = batch_major_ ? 1 : 0;
+  return fwdmi_emb_layer_norm_ex(hipStream, S, B, ld_, static_cast<const int32_t*>(inputs[0]),
+                                 static_cast<const int32_t*>(inputs[1]), static_cast<const int32_t*>(inputs[2]),
+                                 d_params_, d_params_ + ld_, d_word_, d_pos_, d_tok_, t_.word_count, t_.pos_count,
+                                 t_.tok_count, outputs[0], static_cast<int32_t*>(outputs[1]), (int32_t)type_, eps_,
+                                 d_oob_, &ext);
 }
 
 DataType EmbLayerNormPluginDynamic::getOutputDataType(int index, const DataType*, int) const noexcept {
@@ -421,9 +425,10 @@ void EmbLayerNormPluginDynamic::terminate() noexcept {
 // Own layout (the NVIDIA plugin's bytes are not part of the reference tree):
 //   int type | int mha_type | int ld | int word_count | int pos_count | int tok_count | float eps |
 //   beta f32[ld] | gamma f32[ld] | word[word_count*ld] | pos[pos_count*ld] | tok[tok_count*ld]
+// followed, only for a batch-major plugin, by int batch_major(4).
 size_t EmbLayerNormPluginDynamic::getSerializationSize() const noexcept {
   return 6 * sizeof(int32_t) + sizeof(float) + 2 * (size_t)ld_ * sizeof(float) + t_.word->host().size() +
-         t_.pos->host().size() + t_.tok->host().size();
+         t_.pos->host().size() + t_.tok->host().size() + (batch_major_ ? sizeof(int32_t) : 0);
 }
 
 void EmbLayerNormPluginDynamic::serialize(void* buffer) const noexcept {
@@ -440,6 +445,7 @@ void EmbLayerNormPluginDynamic::serialize(void* buffer) const noexcept {
   w.bytes(t_.word->host().data(), t_.word->host().size());
   w.bytes(t_.pos->host().data(), t_.pos->host().size());
   w.bytes(t_.tok->host().data(), t_.tok->host().size());
+  if (batch_major_) w.pod<int32_t>(1);
 }
 
 EmbLayerNormPluginDynamic* EmbLayerNormPluginDynamic::deserialize(const std::string& name, const void* data,
@@ -482,7 +488,9 @@ EmbLayerNormPluginDynamic* EmbLayerNormPluginDynamic::deserialize(const std::str
   t.word = read_table(t.word_count);
   t.pos = read_table(t.pos_count);
   t.tok = read_table(t.tok_count);
-  return new EmbLayerNormPluginDynamic(name, (DataType)type, (DataType)mha, ld, std::move(t), eps);
+  int32_t batch_major = 0;
+  if (r.left() >= sizeof(int32_t)) r.pod(&batch_major);
+  return new EmbLayerNormPluginDynamic(name, (DataType)type, (DataType)mha, ld, std::move(t), eps, batch_major != 0);
 }
 
 void EmbLayerNormPluginDynamic::destroy() noexcept { delete this; }
@@ -499,6 +507,7 @@ EmbLayerNormPluginDynamicCreator::EmbLayerNormPluginDynamicCreator() {
   declare("output_fp16", PluginFieldType::kINT32);
   declare("mha_type_id", PluginFieldType::kINT32);
   declare("eps", PluginFieldType::kFLOAT32);
+  declare("batch_major", PluginFieldType::kINT32);
 }
 
 IPluginV2DynamicExt* EmbLayerNormPluginDynamicCreator::createPlugin(const char* name,
@@ -509,13 +518,14 @@ IPluginV2DynamicExt* EmbLayerNormPluginDynamicCreator::createPlugin(const char* 
     return nullptr;
   }
   std::vector<float> beta, gamma, word, tok, pos;
-  int output_fp16 = 0, mha_type = 0;
+  int output_fp16 = 0, mha_type = 0, batch_major = 0;
   float eps = 0.0f;
   for (int i = 0; i < fc->nbFields; ++i) {
     const PluginField& f = fc->fields[i];
     const std::string n = f.name ? f.name : "";
     bool ok = true;
-    if (n == "bert_embeddings_layernorm_beta") ok = field_to_f32(f, &beta);
+    if (n == "batch_major") ok = f.data && f.type == FWDMI_FIELD_I32, batch_major = ok ? *static_cast<const int*>(f.data) : 0;
+    else if (n == "bert_embeddings_layernorm_beta") ok = field_to_f32(f, &beta);
     else if (n == "bert_embeddings_layernorm_gamma") ok = field_to_f32(f, &gamma);
     else if (n == "bert_embeddings_word_embeddings") ok = field_to_f32(f, &word);
     else if (n == "bert_embeddings_token_type_embeddings") ok = field_to_f32(f, &tok);
@@ -545,7 +555,8 @@ IPluginV2DynamicExt* EmbLayerNormPluginDynamicCreator::createPlugin(const char* 
   t.tok = table_blob(tok, type);
   t.beta = std::move(beta);
   t.gamma = std::move(gamma);
-  auto* p = new EmbLayerNormPluginDynamic(name ? name : "", type, (DataType)mha_type, (int)ld, std::move(t), eps);
+  auto* p = new EmbLayerNormPluginDynamic(name ? name : "", type, (DataType)mha_type, (int)ld, std::move(t), eps,
+                                          batch_major != 0);
   p->setPluginNamespace(mNamespace.c_str());
   return p;
 }

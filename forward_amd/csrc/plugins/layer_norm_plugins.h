@@ -109,7 +109,8 @@ class EmbLayerNormPluginDynamic final : public IPluginV2DynamicExt {
     std::shared_ptr<HostDeviceBlob> word, pos, tok;  // rows in the output type
     int word_count = 0, pos_count = 0, tok_count = 0;
   };
-  EmbLayerNormPluginDynamic(std::string name, DataType type, DataType mha_type, int ld, Tables tables, float eps);
+  EmbLayerNormPluginDynamic(std::string name, DataType type, DataType mha_type, int ld, Tables tables, float eps,
+                            bool batch_major = false);
   static EmbLayerNormPluginDynamic* deserialize(const std::string& name, const void* data, size_t length);
   ~EmbLayerNormPluginDynamic() noexcept override;
 
@@ -141,6 +142,7 @@ class EmbLayerNormPluginDynamic final : public IPluginV2DynamicExt {
   DataType mha_type_;  // type of the attention consumer (kept and serialized, not used here)
   int ld_;
   float eps_;
+  bool batch_major_;  // ids are [B, S] and the output [B, S, H, 1, 1] (no transposes around the plugin)
   Tables t_;
   std::shared_ptr<HostDeviceBlob> params_;  // beta | gamma fp32
   float* d_params_ = nullptr;

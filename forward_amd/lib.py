@@ -33,6 +33,11 @@ class BagExt(C.Structure):
                 ("flags", C.c_int32)]
 
 
+class EmbExt(C.Structure):
+    _fields_ = [("batch_major", C.c_int32), ("eps2", C.c_float), ("skip", C.c_void_p), ("gamma2", C.c_void_p),
+                ("beta2", C.c_void_p), ("bias2", C.c_void_p), ("emb_output", C.c_void_p)]
+
+
 class BagTable(C.Structure):
     _fields_ = [("data", C.c_void_p), ("input", C.c_void_p), ("input_2", C.c_void_p), ("count", C.c_int64),
                 ("input_size", C.c_int64), ("data_offset", C.c_int64), ("out_col", C.c_int64)]
@@ -83,6 +88,8 @@ SIGNATURES = {
     "fwdmi_skip_layer_norm": (C.c_int, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i32, C.c_float]),
     "fwdmi_emb_layer_norm": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32,
                                        _i32, _vp, _vp, _i32, C.c_float, _vp]),
+    "fwdmi_emb_layer_norm_ex": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32,
+                                          _i32, _vp, _vp, _i32, C.c_float, _vp, C.POINTER(EmbExt)]),
     "fwdmi_get_plugin_creator": (_vp, [_cp, _cp]),
     "fwdmi_registry_size": (C.c_int, []),
     "fwdmi_registry_at": (_vp, [C.c_int]),

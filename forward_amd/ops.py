@@ -188,21 +188,42 @@ def layer_norm(x, gamma, beta, bias=None, eps=0.0, out=None, stream=None):
 
 
 def emb_layer_norm(input_ids, segment_ids, input_mask, word, pos, tok, gamma, beta, eps=0.0, oob_flag=None,
-                   out=None, mask_idx=None, stream=None):
-    """ids / mask are int32 ``[S, B]``; returns ``(out [S, B, H], mask_idx int32 [B])``."""
+                   out=None, mask_idx=None, batch_major=False, skip=None, gamma2=None, beta2=None, bias2=None,
+                   eps2=0.0, emb_out=None, stream=None):
+    """BERT embedding + LayerNorm.  ids / mask are int32 ``[S, B]`` (``[B, S]`` with ``batch_major``);
+    returns ``(out, mask_idx int32 [B])`` with ``out`` shaped like the ids plus ``H``.
+
+    ``skip`` (+ ``gamma2``/``beta2``/``bias2``/``eps2``) fuses the SkipLayerNorm that consumes the
+    embedding: ``out = LN2(LN(word+pos+tok) + skip (+ bias2))``; ``emb_out`` also keeps the first stage.
+    """
     ids, seg = _dev(input_ids, "input_ids"), _dev(segment_ids, "segment_ids")
     msk = _dev(input_mask, "input_mask") if input_mask is not None else None
     assert ids.dtype == torch.int32 and seg.dtype == torch.int32 and ids.dim() == 2 and seg.shape == ids.shape
     word, pos, tok = _dev(word, "word"), _dev(pos, "pos"), _dev(tok, "tok")
     assert word.dtype == pos.dtype == tok.dtype
     g, b, _ = _params(gamma, beta)
-    s, bsz = ids.shape
+    s, bsz = (ids.shape[1], ids.shape[0]) if batch_major else ids.shape
     ld = word.shape[1]
     if out is None:
-        out = torch.empty((s, bsz, ld), dtype=word.dtype, device=word.device)
+        out = torch.empty(tuple(ids.shape) + (ld,), dtype=word.dtype, device=word.device)
     if mask_idx is None and msk is not None:
         mask_idx = torch.empty((bsz,), dtype=torch.int32, device=word.device)
-    lib.check(lib.dll.fwdmi_emb_layer_norm(_stream(stream), s, bsz, ld, _p(ids), _p(seg), _p(msk), _p(b), _p(g),
-                                           _p(word), _p(pos), _p(tok), word.shape[0], pos.shape[0], tok.shape[0],
-                                           _p(out), _p(mask_idx), _FDT[word.dtype], eps, _p(oob_flag)))
+    x = lib.EmbExt()
+    x.batch_major = 1 if batch_major else 0
+    keep = []
+    if skip is not None:
+        g2, b2, bias2 = _params(gamma2, beta2, bias2)
+        assert _dev(skip, "skip").dtype == word.dtype and skip.numel() == ids.numel() * ld
+        if emb_out is not None:
+            assert _dev(emb_out, "emb_out").dtype == word.dtype and emb_out.numel() == skip.numel()
+        x.skip, x.gamma2, x.beta2 = skip.data_ptr(), g2.data_ptr(), b2.data_ptr()
+        x.bias2 = bias2.data_ptr() if bias2 is not None else None
+        x.emb_output = emb_out.data_ptr() if emb_out is not None else None
+        x.eps2 = eps2
+        keep = [g2, b2, bias2]
+    lib.check(lib.dll.fwdmi_emb_layer_norm_ex(_stream(stream), s, bsz, ld, _p(ids), _p(seg), _p(msk), _p(b), _p(g),
+                                              _p(word), _p(pos), _p(tok), word.shape[0], pos.shape[0], tok.shape[0],
+                                              _p(out), _p(mask_idx), _FDT[word.dtype], eps, _p(oob_flag),
+                                              C.byref(x)))
+    del keep
     return out, mask_idx

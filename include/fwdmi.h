@@ -181,6 +181,32 @@ int fwdmi_emb_layer_norm(void* stream, int32_t S, int32_t B, int32_t ld, const i
                          int32_t word_count, int32_t pos_count, int32_t tok_count, void* output,
                          int32_t* mask_idx, int32_t dtype, float eps, int32_t* oob_flag);
 
+/*
+ * Options of fwdmi_emb_layer_norm_ex (NULL = the plain call above).
+ *   batch_major: ids / mask are [B, S] and the output is [B, S, ld] (the reference transposes to
+ *     [S, B] before the plugin and back after it, trt_bert_creator.h:64-71,106-109).
+ *   skip != NULL fuses the SkipLayerNorm that consumes the embedding in the same pass:
+ *     first  = LN(word + pos + tok) rounded to `dtype` (also stored to emb_output if given)
+ *     output = LN2(first + skip (+ bias2)) with gamma2 / beta2 / eps2
+ *   which equals fwdmi_emb_layer_norm followed by fwdmi_skip_layer_norm bit for bit.
+ */
+typedef struct fwdmi_emb_ext {
+  int32_t batch_major;
+  float eps2;
+  const void* skip;      /* [rows, ld] in `dtype`, row order as the output */
+  const float* gamma2;   /* fp32 [ld] */
+  const float* beta2;    /* fp32 [ld] */
+  const float* bias2;    /* fp32 [ld] or NULL */
+  void* emb_output;      /* [rows, ld] or NULL */
+} fwdmi_emb_ext;
+
+int fwdmi_emb_layer_norm_ex(void* stream, int32_t S, int32_t B, int32_t ld, const int32_t* input_ids,
+                            const int32_t* segment_ids, const int32_t* input_mask, const float* beta,
+                            const float* gamma, const void* word, const void* pos, const void* tok,
+                            int32_t word_count, int32_t pos_count, int32_t tok_count, void* output,
+                            int32_t* mask_idx, int32_t dtype, float eps, int32_t* oob_flag,
+                            const fwdmi_emb_ext* ext);
+
 /* ========================================================================================= *
  *  2. Plugin objects (opaque handles over the C++ classes in fwdmi_plugin.h)
  * ========================================================================================= */

@@ -202,3 +202,65 @@ def test_launches_can_be_captured_in_a_hip_graph(oracle):
         torch.cuda.synchronize()
         for got, w in zip((emb, midx, out, bag_out), want):
             assert torch.equal(got, w), "replay %d differs from the eager result" % i
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_batch_major_layout_equals_transposed_sequence_major(oracle, dtype):
+    """[B,S] ids in, [B,S,H] out: the transposes the reference wraps around the plugin
+    (trt_bert_creator.h:64-71,106-109) folded into the kernel's indexing."""
+    wl = workloads.config3(variant=11, dtype=dtype, batch=6, seq=40)
+    a = [dev(wl.word), dev(wl.pos), dev(wl.tok), f32(wl.gamma), f32(wl.beta)]
+    ref, rmidx = ops.emb_layer_norm(dev(wl.input_ids), dev(wl.segment_ids), dev(wl.input_mask), *a, eps=wl.eps)
+    t = lambda x: np.ascontiguousarray(x.T)
+    got, midx = ops.emb_layer_norm(dev(t(wl.input_ids)), dev(t(wl.segment_ids)), dev(t(wl.input_mask)), *a,
+                                   eps=wl.eps, batch_major=True)
+    assert tuple(got.shape) == (6, 40, 768)
+    np.testing.assert_array_equal(host(got), host(ref).transpose(1, 0, 2))
+    np.testing.assert_array_equal(host(midx), host(rmidx))
+    np.testing.assert_array_equal(host(midx), wl.valid_len)
+    # through the plugin: optional creator field "batch_major"
+    up = lambda x: x.astype(np.float32)
+    c = REG.getPluginCreator("CustomEmbLayerNormPluginDynamic", "1")
+    p = c.createPlugin("embeddings", [
+        F("bert_embeddings_layernorm_beta", up(wl.beta)), F("bert_embeddings_layernorm_gamma", up(wl.gamma)),
+        F("bert_embeddings_word_embeddings", up(wl.word)), F("bert_embeddings_token_type_embeddings", up(wl.tok)),
+        F("bert_embeddings_position_embeddings", up(wl.pos)), F("output_fp16", int(dtype == np.float16)),
+        F("mha_type_id", 0), F("eps", np.array([wl.eps], np.float32)), F("batch_major", 1)])
+    assert p.getOutputDimensions(0, [(6, 40)] * 3) == [6, 40, 768, 1, 1] and p.getOutputDimensions(1, [(6, 40)] * 3) == [6, 1]
+    e, m = p(dev(t(wl.input_ids)), dev(t(wl.segment_ids)), dev(t(wl.input_mask)))
+    np.testing.assert_array_equal(host(e).reshape(6, 40, 768), host(got))
+    np.testing.assert_array_equal(host(m).reshape(-1), wl.valid_len)
+    q = c.deserializePlugin("embeddings", p.serialize())
+    e2, _ = q(dev(t(wl.input_ids)), dev(t(wl.segment_ids)), dev(t(wl.input_mask)))
+    np.testing.assert_array_equal(host(e2), host(e))
+
+
+@pytest.mark.parametrize("dtype,hidden", [(np.float16, 1024), (np.float32, 1024), (np.float16, 768), (np.float16, 100)])
+def test_fused_emb_skip_equals_two_launches(oracle, dtype, hidden):
+    """One pass computing LN2(LN(word+pos+tok) + residual + bias) is bit-identical to the
+    EmbLayerNorm launch followed by the SkipLayerNorm launch (hidden=100 takes the fallback)."""
+    rng = np.random.Generator(np.random.PCG64(hidden))
+    S, B, V = 48, 5, 300
+    mk = lambda *s, mu=0.0, sd=0.02: (mu + sd * rng.standard_normal(s)).astype(np.float32).astype(dtype)
+    word, pos, tok = mk(V, hidden), mk(64, hidden), mk(2, hidden)
+    g1, b1, g2, b2, bias2 = mk(hidden, mu=1.0), mk(hidden), mk(hidden, mu=1.0), mk(hidden), mk(hidden)
+    ids = rng.integers(0, V, (S, B)).astype(np.int32)
+    seg = rng.integers(0, 2, (S, B)).astype(np.int32)
+    msk = (rng.random((S, B)) < 0.9).astype(np.int32)
+    skip = rng.standard_normal((S, B, hidden)).astype(dtype)
+    common = [dev(ids), dev(seg), dev(msk), dev(word), dev(pos), dev(tok), f32(g1), f32(b1)]
+    emb, midx = ops.emb_layer_norm(*common, eps=1e-12)
+    two = ops.skip_layer_norm(emb, f32(g2), f32(b2), skip=dev(skip), bias=f32(bias2), eps=1e-6)
+    keep = torch.zeros_like(emb)
+    one, midx1 = ops.emb_layer_norm(*common, eps=1e-12, skip=dev(skip), gamma2=f32(g2), beta2=f32(b2),
+                                    bias2=f32(bias2), eps2=1e-6, emb_out=keep)
+    np.testing.assert_array_equal(host(one), host(two))
+    np.testing.assert_array_equal(host(keep), host(emb))
+    np.testing.assert_array_equal(host(midx1), host(midx))
+    # without the optional copy and without bias2
+    two_nb = ops.skip_layer_norm(emb, f32(g2), f32(b2), skip=dev(skip), eps=0.0)
+    one_nb, _ = ops.emb_layer_norm(*common, eps=1e-12, skip=dev(skip), gamma2=f32(g2), beta2=f32(b2))
+    np.testing.assert_array_equal(host(one_nb), host(two_nb))
+    # and against the oracle, stage by stage
+    want = oracle.skip_layer_norm(host(emb), g2, b2, skip=skip, bias=bias2, eps=1e-6)
+    assert_close(host(one), want, dtype)

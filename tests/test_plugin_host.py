@@ -215,5 +215,11 @@ def test_emb_layer_norm_plugin_host_contract():
     assert c.deserializePlugin("e", blob).serialize() == blob and p.clone().serialize() == blob
     with pytest.raises(lib.FwdmiError):
         c.deserializePlugin("e", blob[:-1])
+    # batch-major variant: [B,S] ids, [B,S,H,1,1] output, one trailing int in the blob
+    bm = c.createPlugin("embeddings", fields + [F("batch_major", 1)])
+    assert bm.getOutputDimensions(0, [(4, 12)] * 3) == [4, 12, 16, 1, 1] and bm.getOutputDimensions(1, [(4, 12)] * 3) == [4, 1]
+    bblob = bm.serialize()
+    assert bblob[:-4] == blob and struct.unpack("<i", bblob[-4:]) == (1,)
+    assert c.deserializePlugin("e", bblob).getOutputDimensions(1, [(4, 12)] * 3) == [4, 1]
     with pytest.raises(lib.FwdmiError, match="inconsistent sizes"):
         c.createPlugin("e", fields[:2] + [F("bert_embeddings_word_embeddings", np.zeros(17, np.float32))] + fields[3:])

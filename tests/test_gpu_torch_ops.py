@@ -1,0 +1,62 @@
+"""The PyTorch adapter (torch.ops.fwdmi.* and the drop-in modules) against PyTorch's own
+embedding_bag / embedding on the same device, and a DLRM-style model with its modules swapped."""
+import numpy as np
+import pytest
+import torch
+
+from forward_amd import torch_ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def test_custom_ops_match_torch_on_device():
+    wl = workloads.config2(variant=8, rows=20000, n_bags=500)
+    w, idx, off = (torch.from_numpy(a).cuda() for a in (wl.table, wl.indices.astype(np.int64), wl.offsets.astype(np.int64)))
+    for mode, code in (("sum", 0), ("mean", 1), ("max", 2)):
+        ref = torch.nn.functional.embedding_bag(idx, w, off, mode=mode)
+        got = torch.ops.fwdmi.embedding_bag(w, idx, off, code, None, False)
+        torch.testing.assert_close(got, ref, rtol=1e-5, atol=1e-6)
+    psw = torch.rand(idx.numel(), device="cuda")
+    ref = torch.nn.functional.embedding_bag(idx, w, off, mode="sum", per_sample_weights=psw)
+    torch.testing.assert_close(torch.ops.fwdmi.embedding_bag(w, idx, off, 0, psw, False), ref, rtol=1e-5, atol=1e-6)
+    ids = torch.randint(0, 20000, (7, 3, 5), device="cuda")
+    assert torch.equal(torch.ops.fwdmi.embedding(w, ids), torch.nn.functional.embedding(ids, w))
+    x = torch.randn(9, 4, 768, device="cuda", dtype=torch.float16)
+    sk = torch.randn_like(x)
+    g, b = torch.randn(768, device="cuda"), torch.randn(768, device="cuda")
+    ref = torch.nn.functional.layer_norm((x.float() + sk.float()), (768,), g, b, 1e-5)
+    torch.testing.assert_close(torch.ops.fwdmi.skip_layer_norm(x, sk, g, b, None, 1e-5).float(), ref, rtol=5e-3, atol=1e-2)
+
+
+class TinyDlrm(torch.nn.Module):
+    """Sparse stage of the reference's DLRM test model (test_torch_dlrm.h:34-57): three sum-mode bags, concatenated."""
+
+    def __init__(self, tables):
+        super().__init__()
+        self.emb_l = torch.nn.ModuleList([torch.nn.EmbeddingBag(t.shape[0], t.shape[1], mode="sum") for t in tables])
+        for m, t in zip(self.emb_l, tables):
+            m.weight.data = torch.tensor(t)
+        self.word = torch.nn.Embedding(11, 4)
+
+    def forward(self, offsets, indices, tokens):
+        bags = [m(i, o) for m, i, o in zip(self.emb_l, indices, offsets)]
+        return torch.cat(bags, dim=1), self.word(tokens)
+
+
+def test_swapped_modules_reproduce_the_reference_dlrm_case(kats):
+    d = kats["dlrm"]
+    model = TinyDlrm([np.array(t, np.float32) for t in d["tables"]]).cuda().eval()
+    idx = [torch.tensor(i, device="cuda") for i in d["indices"]]
+    off = [torch.tensor(o, device="cuda") for o in d["offsets"]]
+    tok = torch.tensor([[1, 2, 10], [0, 0, 3]], device="cuda")
+    with torch.no_grad():
+        want_bags, want_tok = model(off, idx, tok)
+        swapped = torch_ops.replace_embedding_modules(model)
+        assert all(isinstance(m, torch_ops.EmbeddingBag) for m in swapped.emb_l) and isinstance(swapped.word, torch_ops.Embedding)
+        got_bags, got_tok = swapped(off, idx, tok)
+    torch.testing.assert_close(got_bags, want_bags, rtol=1e-6, atol=1e-7)
+    assert torch.equal(got_tok, want_tok)
+    expect = np.concatenate([[[0.48071694, 0.18480009], [0.41585842, -0.29087239]],
+                             [[-0.18103497, 0.26449448], [-0.25194445, -0.24395032]],
+                             [[-0.44896644, -0.45899662], [-0.44896644, -0.45899662]]], axis=1)
+    np.testing.assert_allclose(got_bags.cpu().numpy(), expect, atol=1e-4)      # test_torch_dlrm.h:56

@@ -161,8 +161,13 @@ int EmbeddingBagPlugin::enqueue(const PluginTensorDesc* inputDesc, const PluginT
 // "002" bytes:
 //   int dim | int count | int data_offset | int op | int table_dtype | int index_dtype |
 //   int out_dtype | int include_last_offset | int per_sample_weights | size_t n | elem[n]
+// A "002" plugin whose table was given by file (`data_file`) writes, in place of the table,
+//   size_t SIZE_MAX | size_t path_len | path bytes | uint64 byte offset in the file
+// so an engine file stays small and loading maps the table instead of copying it.
 size_t EmbeddingBagPlugin::getSerializationSize() const noexcept {
-  return 4 * sizeof(int) + (version_ext_ ? 5 * sizeof(int) : 0) + sizeof(size_t) + table_->host().size();
+  const size_t head = 4 * sizeof(int) + (version_ext_ ? 5 * sizeof(int) : 0) + sizeof(size_t);
+  if (table_->by_reference()) return head + sizeof(size_t) + table_->path().size() + sizeof(uint64_t);
+  return head + table_->size();
 }
 
 void EmbeddingBagPlugin::serialize(void* buffer) const noexcept {
@@ -178,9 +183,16 @@ void EmbeddingBagPlugin::serialize(void* buffer) const noexcept {
     w.pod<int>(opt_.include_last_offset);
     w.pod<int>(opt_.per_sample_weights);
   }
+  if (table_->by_reference()) {
+    w.pod<size_t>(SIZE_MAX);
+    w.pod<size_t>(table_->path().size());
+    w.bytes(table_->path().data(), table_->path().size());
+    w.pod<uint64_t>(table_->file_offset());
+    return;
+  }
   const size_t es = dtype_size(opt_.table_dtype);
-  w.pod<size_t>(table_->host().size() / es);
-  w.bytes(table_->host().data(), table_->host().size());
+  w.pod<size_t>(table_->size() / es);
+  w.bytes(table_->data(), table_->size());
 }
 
 EmbeddingBagPlugin* EmbeddingBagPlugin::deserialize(const void* data, size_t length, bool version_ext) {
@@ -204,13 +216,39 @@ EmbeddingBagPlugin* EmbeddingBagPlugin::deserialize(const void* data, size_t len
     set_error(FWDMI_ERR_TRUNCATED, "EmbeddingBag: serialized header truncated or malformed");
     return nullptr;
   }
+  if (dim <= 0 || count <= 0 || !is_reduce_op(op)) {
+    set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: serialized fields inconsistent (dim %d, count %d, op %d)", dim, count, op);
+    return nullptr;
+  }
+  const size_t es = dtype_size(opt.table_dtype);
+  {
+    ByteReader peek = r;
+    size_t marker = 0;
+    if (version_ext && peek.pod(&marker) && marker == SIZE_MAX) {   // table by reference
+      size_t path_len = 0;
+      uint64_t file_off = 0;
+      std::string path;
+      bool ok = peek.pod(&path_len) && path_len <= peek.left();
+      if (ok) {
+        path.resize(path_len);
+        ok = peek.bytes(&path[0], path_len) && peek.pod(&file_off);
+      }
+      if (!ok) {
+        set_error(FWDMI_ERR_TRUNCATED, "EmbeddingBag: serialized table reference truncated");
+        return nullptr;
+      }
+      auto blob = HostDeviceBlob::map_file(path, file_off, (size_t)dim * (size_t)count * es);
+      if (!blob) return nullptr;
+      return new EmbeddingBagPlugin(std::move(blob), dim, count, off, static_cast<ReduceOperation>(op), opt, true);
+    }
+  }
   std::vector<uint8_t> bytes;
   size_t n = 0;
-  if (!r.vec(&bytes, dtype_size(opt.table_dtype), &n)) {
+  if (!r.vec(&bytes, es, &n)) {
     set_error(FWDMI_ERR_TRUNCATED, "EmbeddingBag: serialized table truncated");
     return nullptr;
   }
-  if (dim <= 0 || count <= 0 || !is_reduce_op(op) || n != (size_t)dim * (size_t)count) {
+  if (n != (size_t)dim * (size_t)count) {
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: serialized fields inconsistent (dim %d, count %d, op %d, n %zu)",
               dim, count, op, n);
     return nullptr;
@@ -258,6 +296,9 @@ EmbeddingBagPluginCreator::EmbeddingBagPluginCreator(bool version_ext) : version
     declare("output_fp16", PluginFieldType::kINT32);
     declare("include_last_offset", PluginFieldType::kINT32);
     declare("per_sample_weights", PluginFieldType::kINT32);
+    declare("data_file", PluginFieldType::kCHAR);
+    declare("data_file_row_offset", PluginFieldType::kINT32);
+    declare("table_type", PluginFieldType::kINT32);
   }
 }
 
@@ -280,9 +321,10 @@ IPluginV2DynamicExt* EmbeddingBagPluginCreator::createPlugin(const char*, const 
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: expected 5 fields, got %d", fc->nbFields);
     return nullptr;
   }
-  int dim = 0, count = 0, offset = 0, op = -1;
+  int dim = 0, count = 0, offset = 0, op = -1, file_row_offset = 0, table_type = -1;
   bool have[5] = {false, false, false, false, false};
   const PluginField* data = nullptr;
+  std::string data_file;
   EmbeddingBagOptions opt;
   for (int i = 0; i < fc->nbFields; ++i) {
     const PluginField& f = fc->fields[i];
@@ -296,6 +338,8 @@ IPluginV2DynamicExt* EmbeddingBagPluginCreator::createPlugin(const char*, const 
     else if (version_ext_ && name == "include_last_offset") scalar = &opt.include_last_offset;
     else if (version_ext_ && name == "per_sample_weights") scalar = &opt.per_sample_weights;
     else if (version_ext_ && name == "index_type") scalar = &opt.index_dtype;
+    else if (version_ext_ && name == "data_file_row_offset") scalar = &file_row_offset;
+    else if (version_ext_ && name == "table_type") scalar = &table_type;
     if (scalar) {
       if (f.type != FWDMI_FIELD_I32 || !f.data) {
         set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: field '%s' must be INT32", name.c_str());
@@ -309,6 +353,14 @@ IPluginV2DynamicExt* EmbeddingBagPluginCreator::createPlugin(const char*, const 
         return nullptr;
       }
       opt.out_dtype = *static_cast<const int*>(f.data) ? FWDMI_F16 : FWDMI_F32;
+    } else if (version_ext_ && name == "data_file") {
+      if (f.type != FWDMI_FIELD_CHAR || !f.data || f.length <= 0) {
+        set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: field 'data_file' must be a CHAR path");
+        return nullptr;
+      }
+      data_file.assign(static_cast<const char*>(f.data), (size_t)f.length);
+      while (!data_file.empty() && data_file.back() == '\0') data_file.pop_back();
+      have[4] = true;
     } else if (name == "data") {
       const bool type_ok = f.type == FWDMI_FIELD_F32 || (version_ext_ && f.type == FWDMI_FIELD_F16);
       if (!type_ok || !f.data) {
@@ -338,6 +390,19 @@ IPluginV2DynamicExt* EmbeddingBagPluginCreator::createPlugin(const char*, const 
     return nullptr;
   }
   const size_t n = (size_t)dim * (size_t)count;
+  if (!data_file.empty()) {
+    if (data || !is_float_dtype(table_type) || file_row_offset < 0) {
+      set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: 'data_file' excludes 'data' and needs 'table_type' (0 fp32 / 1 fp16)");
+      return nullptr;
+    }
+    opt.table_dtype = table_type;
+    const size_t es = dtype_size(table_type);
+    auto blob = HostDeviceBlob::map_file(data_file, (uint64_t)file_row_offset * dim * es, n * es);
+    if (!blob) return nullptr;
+    auto* obj = new EmbeddingBagPlugin(std::move(blob), dim, count, offset, static_cast<ReduceOperation>(op), opt, true);
+    obj->setPluginNamespace(mNamespace.c_str());
+    return obj;
+  }
   if (data->length >= 0 && (size_t)data->length != n && data->length != 1) {
     // The reference's own field declaration uses length 1 as a placeholder; its caller passes dim*count.
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: 'data' holds %d elements, dim*count = %zu", data->length, n);

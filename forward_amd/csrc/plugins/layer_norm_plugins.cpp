@@ -427,8 +427,8 @@ void EmbLayerNormPluginDynamic::terminate() noexcept {
 //   beta f32[ld] | gamma f32[ld] | word[word_count*ld] | pos[pos_count*ld] | tok[tok_count*ld]
 // followed, only for a batch-major plugin, by int batch_major(4).
 size_t EmbLayerNormPluginDynamic::getSerializationSize() const noexcept {
-  return 6 * sizeof(int32_t) + sizeof(float) + 2 * (size_t)ld_ * sizeof(float) + t_.word->host().size() +
-         t_.pos->host().size() + t_.tok->host().size() + (batch_major_ ? sizeof(int32_t) : 0);
+  return 6 * sizeof(int32_t) + sizeof(float) + 2 * (size_t)ld_ * sizeof(float) + t_.word->size() +
+         t_.pos->size() + t_.tok->size() + (batch_major_ ? sizeof(int32_t) : 0);
 }
 
 void EmbLayerNormPluginDynamic::serialize(void* buffer) const noexcept {
@@ -442,9 +442,9 @@ void EmbLayerNormPluginDynamic::serialize(void* buffer) const noexcept {
   w.pod<float>(eps_);
   w.bytes(t_.beta.data(), t_.beta.size() * 4);
   w.bytes(t_.gamma.data(), t_.gamma.size() * 4);
-  w.bytes(t_.word->host().data(), t_.word->host().size());
-  w.bytes(t_.pos->host().data(), t_.pos->host().size());
-  w.bytes(t_.tok->host().data(), t_.tok->host().size());
+  w.bytes(t_.word->data(), t_.word->size());
+  w.bytes(t_.pos->data(), t_.pos->size());
+  w.bytes(t_.tok->data(), t_.tok->size());
   if (batch_major_) w.pod<int32_t>(1);
 }
 

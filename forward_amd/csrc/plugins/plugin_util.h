@@ -135,23 +135,31 @@ inline void f32_to_f16_bytes(const float* src, size_t n, void* dst) {
 // matter how many times the plugin is cloned.
 class HostDeviceBlob {
  public:
-  explicit HostDeviceBlob(std::vector<uint8_t> host) : host_(std::move(host)) {}
-  ~HostDeviceBlob() {
-    if (dev_) (void)hipFree(dev_);
+  explicit HostDeviceBlob(std::vector<uint8_t> host) : host_(std::move(host)) {
+    data_ = host_.data();
+    size_ = host_.size();
   }
+  // A read-only mapping of `nbytes` of `path` starting at `offset`: the table stays in the
+  // page cache instead of being copied into the process (and into every serialized engine).
+  static std::shared_ptr<HostDeviceBlob> map_file(const std::string& path, uint64_t offset, size_t nbytes);
+  ~HostDeviceBlob();
   HostDeviceBlob(const HostDeviceBlob&) = delete;
   HostDeviceBlob& operator=(const HostDeviceBlob&) = delete;
 
-  const std::vector<uint8_t>& host() const { return host_; }
+  const uint8_t* data() const { return data_; }
+  size_t size() const { return size_; }
+  bool by_reference() const { return !path_.empty(); }
+  const std::string& path() const { return path_; }
+  uint64_t file_offset() const { return file_offset_; }
   // Takes a device reference, uploading on first use.  Returns a status.
   int acquire(void** dev) {
     std::lock_guard<std::mutex> lock(mu_);
     if (!dev_) {
-      const size_t n = host_.empty() ? 16 : host_.size();
+      const size_t n = size_ ? size_ : 16;
       void* p = nullptr;
       FWDMI_HIP_CHECK(hipMalloc(&p, n));
-      if (!host_.empty()) {
-        hipError_t e = hipMemcpy(p, host_.data(), host_.size(), hipMemcpyHostToDevice);
+      if (size_) {
+        hipError_t e = hipMemcpy(p, data_, size_, hipMemcpyHostToDevice);
         if (e != hipSuccess) {
           (void)hipFree(p);
           return set_error(FWDMI_ERR_HIP, "hipMemcpy (table upload) failed: %s", hipGetErrorString(e));
@@ -172,7 +180,14 @@ class HostDeviceBlob {
   }
 
  private:
+  HostDeviceBlob() = default;
   std::vector<uint8_t> host_;
+  const uint8_t* data_ = nullptr;
+  size_t size_ = 0;
+  std::string path_;       // non-empty: data_ points into a file mapping
+  uint64_t file_offset_ = 0;
+  void* map_base_ = nullptr;
+  size_t map_len_ = 0;
   std::mutex mu_;
   void* dev_ = nullptr;
   int users_ = 0;

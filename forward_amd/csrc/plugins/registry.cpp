@@ -1,6 +1,11 @@
 // Process-wide plugin registry: creators are looked up by (name, version, namespace), the way
 // the reference's layer creators find theirs (getPluginRegistry()->getPluginCreator(...),
 // source/trt_engine/trt_network_crt/layer_creators/trt_embedding_bag_creator.h:54-55).
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
 #include <mutex>
 #include <string>
 #include <vector>
@@ -46,6 +51,43 @@ class PluginRegistry final : public IPluginRegistry {
 };
 
 }  // namespace
+
+HostDeviceBlob::~HostDeviceBlob() {
+  if (dev_) (void)hipFree(dev_);
+  if (map_base_) munmap(map_base_, map_len_);
+}
+
+std::shared_ptr<HostDeviceBlob> HostDeviceBlob::map_file(const std::string& path, uint64_t offset, size_t nbytes) {
+  const int fd = open(path.c_str(), O_RDONLY);
+  if (fd < 0) {
+    set_error(FWDMI_ERR_BAD_ARG, "cannot open table file '%s'", path.c_str());
+    return nullptr;
+  }
+  struct stat st {};
+  if (fstat(fd, &st) != 0 || (uint64_t)st.st_size < offset + nbytes) {
+    close(fd);
+    set_error(FWDMI_ERR_TRUNCATED, "table file '%s' is shorter than offset %llu + %zu bytes", path.c_str(),
+              (unsigned long long)offset, nbytes);
+    return nullptr;
+  }
+  const uint64_t page = (uint64_t)sysconf(_SC_PAGESIZE);
+  const uint64_t base = offset / page * page;
+  const size_t len = (size_t)(offset - base) + nbytes;
+  void* m = len ? mmap(nullptr, len, PROT_READ, MAP_PRIVATE, fd, (off_t)base) : nullptr;
+  close(fd);
+  if (len && m == MAP_FAILED) {
+    set_error(FWDMI_ERR_BAD_ARG, "mmap of table file '%s' failed", path.c_str());
+    return nullptr;
+  }
+  std::shared_ptr<HostDeviceBlob> b(new HostDeviceBlob());
+  b->path_ = path;
+  b->file_offset_ = offset;
+  b->map_base_ = m;
+  b->map_len_ = len;
+  b->data_ = static_cast<const uint8_t*>(m) + (offset - base);
+  b->size_ = nbytes;
+  return b;
+}
 
 IPluginRegistry* getPluginRegistry() noexcept {
   static PluginRegistry registry;

@@ -119,6 +119,13 @@ SIGNATURES = {
     "fwdmi_plugin_clone": (_vp, [_vp]),
     "fwdmi_plugin_destroy": (None, [_vp]),
     "fwdmi_plugin_take_oob_flag": (C.c_int, [_vp, _vp]),
+    "fwdmi_plan_save": (C.c_int, [_cp, C.POINTER(_vp), C.POINTER(_cp), C.c_int, _cp]),
+    "fwdmi_plan_load": (_vp, [_cp]),
+    "fwdmi_plan_size": (C.c_int, [_vp]),
+    "fwdmi_plan_layer_name": (_cp, [_vp, C.c_int]),
+    "fwdmi_plan_take_plugin": (_vp, [_vp, C.c_int]),
+    "fwdmi_plan_meta": (_cp, [_vp]),
+    "fwdmi_plan_close": (None, [_vp]),
 }
 
 

@@ -211,3 +211,35 @@ class PluginRegistry:
 
 def getPluginRegistry():
     return PluginRegistry()
+
+
+# Keys of the reference's engine sidecar (source/trt_engine/trt_common/trt_meta_data.cpp:42-97).
+META_KEYS = ("infer_mode", "max_batch_size", "opt_batch_size", "output_indices", "unused_input_indices",
+             "torch_module_path")
+
+
+def save_plan(path, layers, meta=None):
+    """Writes ``layers`` = [(layer_name, Plugin), ...] to ``path`` and ``meta`` (a dict with the
+    reference's sidecar keys) to ``path + ".meta"``: the plugin part of ``TrtForwardEngine::Save``."""
+    import json
+    n = len(layers)
+    handles = (C.c_void_p * max(1, n))(*[p._h for _, p in layers])
+    names = (C.c_char_p * max(1, n))(*[name.encode() for name, _ in layers])
+    text = None if meta is None else json.dumps(meta).encode()
+    lib.check(lib.dll.fwdmi_plan_save(path.encode(), handles, names, n, text))
+
+
+def load_plan(path):
+    """Returns ``([(layer_name, Plugin), ...], meta_dict)``: the plugin part of ``TrtForwardEngine::Load``."""
+    import json
+    h = lib.dll.fwdmi_plan_load(path.encode())
+    if not h:
+        raise lib.FwdmiError(lib.ERR_TRUNCATED, lib.last_error())
+    h = C.c_void_p(h)
+    try:
+        layers = [(lib.dll.fwdmi_plan_layer_name(h, i).decode(), Plugin(lib.dll.fwdmi_plan_take_plugin(h, i)))
+                  for i in range(lib.dll.fwdmi_plan_size(h))]
+        text = lib.dll.fwdmi_plan_meta(h).decode()
+    finally:
+        lib.dll.fwdmi_plan_close(h)
+    return layers, (json.loads(text) if text else {})

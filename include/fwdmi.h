@@ -285,6 +285,31 @@ void fwdmi_plugin_destroy(fwdmi_plugin* p);
  * stream; diagnostic, not part of the reference contract). Returns 0/1 or a negative status. */
 int fwdmi_plugin_take_oob_flag(fwdmi_plugin* p, void* stream);
 
+/* ========================================================================================= *
+ *  3. Plan files: the plugins of an engine in one file + the "<file>.meta" JSON sidecar
+ *     replaces the plugin part of TrtForwardEngine::Save / Load
+ *     (source/trt_engine/trt_engine/trt_fwd_engine.cpp:156-209) and the sidecar of
+ *     source/trt_engine/trt_common/trt_meta_data.cpp:42-97 (keys infer_mode, max_batch_size,
+ *     opt_batch_size, output_indices, unused_input_indices, torch_module_path; the text is
+ *     stored as given).
+ * ========================================================================================= */
+typedef struct fwdmi_plan fwdmi_plan;
+
+/* Serializes n plugins (with the layer names they were created under) into `path`;
+ * meta_json (may be NULL) goes to "<path>.meta". */
+int fwdmi_plan_save(const char* path, fwdmi_plugin* const* plugins, const char* const* layer_names, int n,
+                    const char* meta_json);
+/* Reads a plan back: every entry is re-created through its registered creator's
+ * deserializePlugin.  NULL on a missing / truncated file or an unknown (type, version). */
+fwdmi_plan* fwdmi_plan_load(const char* path);
+int fwdmi_plan_size(fwdmi_plan* plan);
+const char* fwdmi_plan_layer_name(fwdmi_plan* plan, int i);
+/* Hands entry i to the caller (who destroys it); a second call for the same i returns NULL. */
+fwdmi_plugin* fwdmi_plan_take_plugin(fwdmi_plan* plan, int i);
+/* Text of "<path>.meta" ("" if the sidecar is absent). */
+const char* fwdmi_plan_meta(fwdmi_plan* plan);
+void fwdmi_plan_close(fwdmi_plan* plan);
+
 #ifdef __cplusplus
 }
 #endif

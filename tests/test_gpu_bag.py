@@ -248,3 +248,109 @@ def test_plugin_modes_fixed_gather_and_extended(oracle):
     assert got.dtype == np.float16 and got.shape == (200, 128)
     assert_bits_equal(got, want, "extended plugin")
     assert not p.takeOobFlag()
+
+
+def test_large_tables_and_offsets_take_the_wide_address_path(oracle):
+    """int32 ids normally use 24-bit row arithmetic; these shapes must fall back to 64-bit:
+    more than 2^24 rows, a table larger than 4 GiB, a negative data_offset, ids near 2^31."""
+    rng = np.random.Generator(np.random.PCG64(91))
+    rows = (1 << 24) + 4096                                        # > 2^24 rows of 16 bytes
+    table = torch.empty((rows, 8), dtype=torch.float16, device="cuda")
+    table.copy_(((torch.arange(rows, device="cuda") % 2039).float() / 64).unsqueeze(1)
+                + torch.arange(8, device="cuda").float() / 512)
+    lengths = rng.integers(0, 7, 200)
+    idx = rng.integers(rows - 5000, rows, int(lengths.sum())).astype(np.int32)   # the top of the table
+    idx[::3] = rng.integers(0, 1000, idx[::3].size)
+    off = workloads.offsets_from_lengths(lengths, np.int32)
+    got = host(ops.embedding_bag(table, dev(idx), dev(off), "sum"))
+    uniq, inv = np.unique(idx, return_inverse=True)
+    sub = host(table[torch.from_numpy(uniq.astype(np.int64)).cuda()])
+    want, _, _ = oracle.embedding_bag(sub, inv.astype(np.int32), off, oracle.OP_SUM)
+    assert_bits_equal(got, want, "2^24+ rows")
+    del table
+
+    big_rows = 2_200_000                                           # 2.2 M rows x 2 KiB = 4.5 GB > 4 GiB
+    big = torch.empty((big_rows, 512), dtype=torch.float32, device="cuda")
+    big.copy_((torch.arange(big_rows, device="cuda") % 4093).float().unsqueeze(1) / 8
+              + torch.arange(512, device="cuda").float() / 1024)
+    idx = rng.integers(big_rows - 3000, big_rows, int(lengths.sum())).astype(np.int32)
+    got = host(ops.embedding_bag(big, dev(idx), dev(off), "sum"))
+    uniq, inv = np.unique(idx, return_inverse=True)
+    sub = host(big[torch.from_numpy(uniq.astype(np.int64)).cuda()])
+    want, _, _ = oracle.embedding_bag(sub, inv.astype(np.int32), off, oracle.OP_SUM)
+    assert_bits_equal(got, want, "table beyond 4 GiB")
+    del big
+
+    small = rng.standard_normal((64, 16)).astype(np.float32)
+    for data_offset in (-20, 2**31 - 40):                          # id range leaves [0, 2^31)
+        ids = (rng.integers(0, 64, 300) + data_offset).astype(np.int64)
+        ids[::7] = data_offset - 1                                 # just below the shard: skipped
+        ids32 = np.clip(ids, -2**31, 2**31 - 1).astype(np.int32)
+        o = workloads.offsets_from_lengths(np.full(30, 10), np.int32)
+        got = host(ops.embedding_bag(dev(small), dev(ids32), dev(o), "sum", data_offset=data_offset))
+        want, _, oob = oracle.embedding_bag(small, ids32, o, oracle.OP_SUM, data_offset=data_offset)
+        assert oob > 0
+        assert_bits_equal(got, want, "data_offset %d" % data_offset)
+
+
+def test_malformed_offsets_stay_in_bounds():
+    """Offsets that decrease, exceed the id count or are negative are clamped; nothing is read or
+    written out of bounds and well-formed bags of the same batch are still right."""
+    rng = np.random.Generator(np.random.PCG64(92))
+    table = rng.standard_normal((100, 32)).astype(np.float32)
+    idx = rng.integers(0, 100, 50).astype(np.int32)
+    off = np.array([0, 10, 5, 20, 1000, -7, 30, 40], np.int32)     # bag 1 "ends" before it starts, etc.
+    guard = torch.full((8 + 2, 32), 123.0, device="cuda")
+    out = guard[1:9]
+    ops.embedding_bag(dev(table), dev(idx), dev(off), "sum", out=out)
+    torch.cuda.synchronize()
+    got = guard.cpu().numpy()
+    assert (got[0] == 123.0).all() and (got[9] == 123.0).all()     # rows around the output untouched
+    np.testing.assert_allclose(got[1], table[idx[0:10]].sum(0), rtol=1e-5, atol=1e-5)   # bag 0 = ids 0..10
+    np.testing.assert_array_equal(got[2], 0.0)                                         # 10..5 -> empty
+    np.testing.assert_allclose(got[3], table[idx[5:20]].sum(0), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(got[4], table[idx[20:50]].sum(0), rtol=1e-5, atol=1e-5)  # 20..1000 -> 20..50
+    np.testing.assert_array_equal(got[5], 0.0)                                         # 50..0 -> empty
+    np.testing.assert_allclose(got[6], table[idx[0:30]].sum(0), rtol=1e-5, atol=1e-5)   # -7 -> 0
+    np.testing.assert_allclose(got[8], table[idx[40:50]].sum(0), rtol=1e-5, atol=1e-5)  # last bag runs to the end
+    assert np.isfinite(got).all()
+
+
+def test_concurrent_enqueue_from_threads_on_their_own_streams(oracle):
+    """enqueue is re-entrant across plugin instances and stream-ordered: four host threads, each
+    with its own stream and its own clone of one plugin, interleave launches."""
+    import threading
+    wl = workloads.config2(variant=12, rows=8000, n_bags=1500)
+    want, _, _ = oracle.embedding_bag(wl.table, wl.indices, wl.offsets, oracle.OP_SUM)
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    base = c.createPlugin("embedding_bag", bag_fields(wl.table))
+    idx, off = dev(wl.indices), dev(wl.offsets)
+    io_in = [((wl.indices.size,), lib.I32), ((wl.n_bags,), lib.I32)]
+    io_out = [((wl.n_bags, 128), lib.F32)]
+    base.configurePlugin(io_in, io_out)
+    results, errors = {}, []
+
+    def work(k):
+        try:
+            p = base.clone()
+            p.configurePlugin(io_in, io_out)
+            s = torch.cuda.Stream()
+            outs = [torch.empty((wl.n_bags, 128), device="cuda") for _ in range(10)]
+            for o in outs:
+                p.enqueue([idx, off], [o], stream=s)
+            s.synchronize()
+            results[k] = [host(o) for o in outs]
+            p.destroy()
+        except Exception as e:       # pragma: no cover
+            errors.append(e)
+
+    torch.cuda.synchronize()
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for k in range(4):
+        for got in results[k]:
+            assert_bits_equal(got, want, "thread %d" % k)

@@ -223,3 +223,40 @@ def test_emb_layer_norm_plugin_host_contract():
     assert c.deserializePlugin("e", bblob).getOutputDimensions(1, [(4, 12)] * 3) == [4, 1]
     with pytest.raises(lib.FwdmiError, match="inconsistent sizes"):
         c.createPlugin("e", fields[:2] + [F("bert_embeddings_word_embeddings", np.zeros(17, np.float32))] + fields[3:])
+
+
+def test_creators_and_plugins_are_thread_safe():
+    """Build-time calls from several host threads at once (ctypes releases the GIL): creators are
+    shared registry objects, plugins and their clones share table storage."""
+    import threading
+    c = REG.getPluginCreator("EmbeddingBag_TRT", "001")
+    shared = c.createPlugin("shared", bag_fields(np.arange(200, dtype=np.float32).reshape(50, 4)))
+    want = shared.serialize()
+    errors = []
+
+    def work(seed):
+        try:
+            rng = np.random.default_rng(seed)
+            for _ in range(30):
+                t = rng.standard_normal((int(rng.integers(1, 40)), 8)).astype(np.float32)
+                p = c.createPlugin("t%d" % seed, bag_fields(t))
+                blob = p.serialize()
+                assert blob[24:] == t.tobytes()
+                q = c.deserializePlugin("t", blob)
+                assert q.getOutputDimensions(0, [(9,), (3,)]) == [3, 8]
+                k = shared.clone()
+                assert k.serialize() == want
+                with pytest.raises(lib.FwdmiError, match="expected 5 fields"):
+                    c.createPlugin("bad", bag_fields(t)[:3])       # error text is per thread
+                for o in (p, q, k):
+                    o.destroy()
+        except Exception as e:       # pragma: no cover
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(s,)) for s in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert shared.serialize() == want

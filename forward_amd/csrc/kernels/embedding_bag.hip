@@ -234,10 +234,11 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     // folds them in bag order.  LDS selects where the ids come from.  COMPACT selects 32-bit
     // arithmetic: ids are int32, every in-range id is non-negative, the table has at most 2^24
     // rows and 4 GiB, so a row's byte offset is one 24-bit multiply-add on top of a uniform base.
-    auto step = [&](auto uu_tag, auto lds_tag, auto compact_tag, int64_t i) {
+    auto step = [&](auto uu_tag, auto lds_tag, auto compact_tag, auto pred_tag, int64_t i, int cnt) {
       constexpr int UU = decltype(uu_tag)::value;
       constexpr bool LDS = decltype(lds_tag)::value;
       constexpr bool COMPACT = decltype(compact_tag)::value;
+      constexpr bool PRED = decltype(pred_tag)::value;  // only the first `cnt` of the UU rows exist
       Pack<TW, VEC> v[UU];
       TI id[UU];
       float w[UU];
@@ -250,42 +251,64 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
         const float* const wp = s_w + li;
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
-          id[u] = sp[u];
-          if (KIND == kWeighted) w[u] = wp[u];
+          id[u] = 0;
+          w[u] = 0.0f;
+          if (!PRED || u < cnt) {
+            id[u] = sp[u];
+            if (KIND == kWeighted) w[u] = wp[u];
+          }
         }
       } else {
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
-          id[u] = ids[i + u];
-          if (KIND == kWeighted) w[u] = (float)psw[i + u];
+          id[u] = 0;
+          w[u] = 0.0f;
+          if (!PRED || u < cnt) {
+            id[u] = ids[i + u];
+            if (KIND == kWeighted) w[u] = (float)psw[i + u];
+          }
         }
       }
-      // a bad id never forms an address: a valid row is fetched instead and discarded below
+      // a bad id never forms an address: a valid row is fetched instead and discarded below;
+      // rows past `cnt` are not fetched at all and enter the fold as zeros
       if (COMPACT) {
         uint32_t worst = 0;
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
-          const uint32_t row = (uint32_t)id[u] - lo32;
+          const bool valid = !PRED || u < cnt;
+          const uint32_t row = valid ? (uint32_t)id[u] - lo32 : 0u;
           worst = max(worst, row);
           const uint32_t off = __umul24(min(row, last32), row_bytes) + col_bytes;
-          v[u] = gload<TW, VEC>(reinterpret_cast<const TW FWDMI_GLOBAL*>(tab_bytes + off));
-          if (KIND == kMax) ok[u] = row <= last32;
+          if (valid) {
+            v[u] = gload<TW, VEC>(reinterpret_cast<const TW FWDMI_GLOBAL*>(tab_bytes + off));
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[u].v[e] = (TW)0.0f;
+          }
+          if (KIND == kMax) ok[u] = valid && row <= last32;
         }
         all_ok = worst <= last32;
       } else {
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
+          const bool valid = !PRED || u < cnt;
           const uint64_t row = (uint64_t)((int64_t)id[u] - T.data_offset);
-          ok[u] = row < (uint64_t)T.count;
-          v[u] = gload<TW, VEC>(tcol + (ok[u] ? row : 0) * (uint64_t)L.dim);
-          all_ok &= ok[u];
+          const bool in_range = row < (uint64_t)T.count;
+          ok[u] = valid && in_range;
+          if (valid) {
+            v[u] = gload<TW, VEC>(tcol + (in_range ? row : 0) * (uint64_t)L.dim);
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[u].v[e] = (TW)0.0f;
+          }
+          all_ok &= in_range || !valid;
         }
       }
       if (__builtin_expect(!__all(all_ok), 0)) {
         oob |= !all_ok;
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
-          if (COMPACT) ok[u] = ((uint32_t)id[u] - lo32) <= last32;
+          if (COMPACT) ok[u] = (!PRED || u < cnt) && ((uint32_t)id[u] - lo32) <= last32;
           if (!ok[u]) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) v[u].v[e] = (TW)0.0f;
@@ -322,16 +345,12 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     };
     auto bag = [&](auto lds_tag, auto compact_tag) {
       int64_t i = start;
-      for (; i + kUnroll <= end; i += kUnroll) step(std::integral_constant<int, kUnroll>{}, lds_tag, compact_tag, i);
-      if (i + 4 <= end) {
-        step(std::integral_constant<int, 4>{}, lds_tag, compact_tag, i);
-        i += 4;
-      }
-      if (i + 2 <= end) {
-        step(std::integral_constant<int, 2>{}, lds_tag, compact_tag, i);
-        i += 2;
-      }
-      if (i < end) step(std::integral_constant<int, 1>{}, lds_tag, compact_tag, i);
+      for (; i + kUnroll <= end; i += kUnroll)
+        step(std::integral_constant<int, kUnroll>{}, lds_tag, compact_tag, std::false_type{}, i, kUnroll);
+      // the last 1..7 rows: one predicated step, so a wavefront issues as many loads as its
+      // longest remainder needs and no more
+      if (i < end)
+        step(std::integral_constant<int, kUnroll - 1>{}, lds_tag, compact_tag, std::true_type{}, i, (int)(end - i));
     };
     if (in_lds) {
       if (compact)

@@ -136,6 +136,8 @@ int EmbeddingBagPlugin::enqueue(const PluginTensorDesc* inputDesc, const PluginT
     return set_error(FWDMI_ERR_UNSUPPORTED, "Unsupported input data type %d", inputDesc[0].type);
 
   const Dims& in0 = inputDesc[0].dims;
+  if (in0.nbDims != 1 && in0.nbDims != 2)
+    return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag::enqueue: ids must be 1-D or 2-D, got %d-D", in0.nbDims);
   if (in0.nbDims > 1) {
     const int64_t batch_size = in0.d[0], bag_len = in0.d[1];
     const fwdmi_bag_ext x = make_ext(opt_, nullptr, d_oob_);
@@ -149,6 +151,8 @@ int EmbeddingBagPlugin::enqueue(const PluginTensorDesc* inputDesc, const PluginT
     return set_error(FWDMI_ERR_UNSUPPORTED, "EmbeddingBag: GATHER with an offsets input is not supported");
   const int64_t input_size = in0.d[0];
   const Dims& in1 = inputDesc[1].dims;
+  if (!(in1.nbDims == 1 || (in1.nbDims == 2 && in1.d[0] == 1)))
+    return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag::enqueue: offsets must be [B] or [1, B]");
   const int64_t n_off = in1.nbDims == 1 ? in1.d[0] : in1.d[1];
   const int64_t n_bags = n_off - (opt_.include_last_offset ? 1 : 0);
   const fwdmi_bag_ext x = make_ext(opt_, opt_.per_sample_weights ? inputs[2] : nullptr, d_oob_);
@@ -403,8 +407,10 @@ IPluginV2DynamicExt* EmbeddingBagPluginCreator::createPlugin(const char*, const 
     obj->setPluginNamespace(mNamespace.c_str());
     return obj;
   }
-  if (data->length >= 0 && (size_t)data->length != n && data->length != 1) {
-    // The reference's own field declaration uses length 1 as a placeholder; its caller passes dim*count.
+  if (data->length < 0 || (size_t)data->length != n) {
+    // The reference copies dim*count floats whatever the field's length says
+    // (embedding_bag_plugin.cpp:283-285); its caller passes dim*count
+    // (trt_embedding_bag_creator.h:62-64).  Anything else would read past the caller's array.
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: 'data' holds %d elements, dim*count = %zu", data->length, n);
     return nullptr;
   }

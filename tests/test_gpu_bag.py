@@ -215,6 +215,11 @@ def test_plugin_serialize_load_run_matches(oracle):
     # wrong id type is refused with -1, as in the reference
     rc = p.enqueue_raw([((idx.size,), lib.I64), ((64,), lib.I64)], [((64, 64), lib.F32)], [0, 0], [0])
     assert rc == lib.ERR_UNSUPPORTED
+    # shapes the plugin's own shape rules never produce are refused before any launch
+    rc = p.enqueue_raw([((4, 4, 4), lib.I32)], [((4, 64), lib.F32)], [0], [0])
+    assert rc == lib.ERR_BAD_ARG and "1-D or 2-D" in lib.last_error()
+    rc = p.enqueue_raw([((idx.size,), lib.I32), ((2, 32), lib.I32)], [((64, 64), lib.F32)], [0, 0], [0])
+    assert rc == lib.ERR_BAD_ARG and "offsets" in lib.last_error()
 
 
 def test_plugin_modes_fixed_gather_and_extended(oracle):

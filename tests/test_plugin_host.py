@@ -46,6 +46,8 @@ def test_embedding_bag_creator_fields():
         c.createPlugin("x", bag_fields(table)[:4] + [F("data", table.astype(np.float16))])
     with pytest.raises(lib.FwdmiError, match="dim\\*count"):
         c.createPlugin("x", bag_fields(table)[:4] + [F("data", table[:3])])
+    with pytest.raises(lib.FwdmiError, match="dim\\*count"):           # a 1-element placeholder is not a table
+        c.createPlugin("x", bag_fields(table)[:4] + [F("data", table[:1, :1])])
 
 
 def test_embedding_bag_output_dimensions_and_formats():

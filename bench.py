@@ -35,7 +35,8 @@ def parse():
     ap.add_argument("--tables", type=int, default=26, help="debug only: fewer tables (not the named config)")
     ap.add_argument("--bags", type=int, default=65536, help="debug only: smaller batch (not the named config)")
     ap.add_argument("--per-table", action="store_true", help="26 launches instead of the fused one")
-    ap.add_argument("--xcd-affinity", action="store_true", help="fused launch with per-XCD table affinity")
+    ap.add_argument("--no-xcd-affinity", action="store_true",
+                    help="fused launch without per-XCD table affinity (every XCD works on every table)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     ap.add_argument("--no-extra", action="store_true", help="skip the config 2/3/5 side measurements")
     ap.add_argument("--cpu-bags", type=int, default=4096, help="bags per table in the CPU baseline sample")
@@ -261,7 +262,7 @@ def main():
         launches_per_step = batch.n_tables
     else:
         def step():
-            batch.forward(out=out, xcd_table_affinity=args.xcd_affinity)
+            batch.forward(out=out, xcd_table_affinity=not args.no_xcd_affinity)
         launches_per_step = 1
 
     wall, per = time_events(torch, step, args.steps, args.warmup)
@@ -281,7 +282,8 @@ def main():
                                % (len(wl.rows), wl.n_bags, wl.dim, wl.n_indices() / total_bags, wl.n_bags,
                                   batch.width, "" if (args.tables == 26 and args.bags == 65536) else " (REDUCED, debug)"),
                    "storage": "fp16 rows and output, fp32 accumulation, int32 ids",
-                   "launch": "per-table" if args.per_table else "fused multi-table",
+                   "launch": "per-table" if args.per_table else
+                   ("fused multi-table" if args.no_xcd_affinity else "fused multi-table, per-XCD table affinity"),
                    "total_ids": wl.n_indices(), "table_bytes": int(sum(t.numel() * 2 for t in tabs))},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,

@@ -30,7 +30,7 @@ class BagExt(C.Structure):
     _fields_ = [("table_dtype", C.c_int32), ("index_dtype", C.c_int32), ("out_dtype", C.c_int32),
                 ("include_last_offset", C.c_int32), ("per_sample_weights", C.c_void_p),
                 ("max_indices", C.c_void_p), ("out_row_stride", C.c_int64), ("oob_flag", C.c_void_p),
-                ("flags", C.c_int32)]
+                ("flags", C.c_int32), ("table_cost", C.c_void_p)]
 
 
 class EmbExt(C.Structure):
@@ -83,6 +83,7 @@ SIGNATURES = {
     "fwdmi_embedding_bag": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _i32, _i64, _i32, C.POINTER(BagExt), _vp]),
     "fwdmi_embedding_bag_fixed": (C.c_int, [_vp, _vp, _i64, _i64, _vp, _i64, _i32, _i64, _i32, C.POINTER(BagExt), _vp]),
     "fwdmi_gather": (C.c_int, [_vp, _vp, _i64, _i64, _vp, _i64, _i32, _i64, C.POINTER(BagExt), _vp]),
+    "fwdmi_bag_table_cost": (C.c_int, [_vp, _i32, _vp]),
     "fwdmi_embedding_bag_multi": (C.c_int, [_vp, _i32, _i64, _vp, _i32, _i32, C.c_double, C.POINTER(BagExt), _vp]),
     "fwdmi_layer_norm": (C.c_int, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _i32, C.c_float]),
     "fwdmi_skip_layer_norm": (C.c_int, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i32, C.c_float]),

@@ -38,7 +38,7 @@ def _op(mode):
 
 
 def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_indices=None, out_row_stride=0,
-         oob_flag=None, flags=0):
+         oob_flag=None, flags=0, table_cost=None):
     x = lib.BagExt()
     x.table_dtype = _FDT[table.dtype]
     x.index_dtype = _IDT[indices.dtype]
@@ -49,6 +49,7 @@ def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_ind
     x.out_row_stride = int(out_row_stride)
     x.oob_flag = oob_flag.data_ptr() if oob_flag is not None else None
     x.flags = flags
+    x.table_cost = table_cost.ctypes.data if table_cost is not None else None
     return x
 
 
@@ -141,14 +142,27 @@ class MultiTableBatch:
         self.total_indices = int(sum(i.numel() for i in self.indices))
         self.desc = torch.from_numpy(desc).to(self.tables[0].device)
 
-    def forward(self, out=None, mode="sum", out_dtype=None, oob_flag=None, xcd_table_affinity=False, stream=None):
+    def default_table_cost(self):
+        """The library's per-table cost estimate for the XCD segmentation (from the table sizes)."""
+        nbytes = np.array([t.numel() * t.element_size() for t in self.tables], np.int64)
+        cost = np.empty(self.n_tables, np.float32)
+        lib.check(lib.dll.fwdmi_bag_table_cost(nbytes.ctypes.data, self.n_tables, cost.ctypes.data))
+        return cost
+
+    def forward(self, out=None, mode="sum", out_dtype=None, oob_flag=None, xcd_table_affinity=False, stream=None,
+                table_cost=None):
         odt = self.tables[0].dtype if out_dtype is None else out_dtype
         if out is None:
             out = torch.empty((self.n_bags, self.width), dtype=odt, device=self.desc.device)
         _dev(out, "out")
         assert out.dtype == odt and out.shape[0] == self.n_bags and out.shape[1] >= self.width
+        cost = None
+        if xcd_table_affinity:
+            cost = self.default_table_cost() if table_cost is None else table_cost
+            cost = np.ascontiguousarray(cost, np.float32)
+            assert cost.shape == (self.n_tables,)
         x = _ext(self.tables[0], self.indices[0], odt, out_row_stride=out.shape[1], oob_flag=oob_flag,
-                 flags=lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0)
+                 flags=lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0, table_cost=cost)
         avg = self.total_indices / max(1, self.n_bags * self.n_tables)
         lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(self.desc), self.n_tables, self.n_bags, _p(out), self.dim,
                                                     _op(mode), avg, C.byref(x), _stream(stream)))

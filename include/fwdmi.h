@@ -87,11 +87,15 @@ typedef struct fwdmi_bag_ext {
   int32_t* oob_flag;           /* device int, set to 1 (sticky) when an id falls outside
                                   [data_offset, data_offset+count); may be NULL */
   int32_t flags;               /* FWDMI_BAG_* bits, 0 for none */
+  const float* table_cost;     /* HOST array [n_tables] or NULL: relative cost of one bag of each
+                                  table, used by FWDMI_BAG_XCD_TABLE_AFFINITY */
 } fwdmi_bag_ext;
 
 /* Multi-table launches only: renumber workgroups so that each of the 8 XCDs (one L2 each)
- * works through whole tables.  Cuts L2 fill traffic; off by default because on the 26-table
- * configuration the uneven per-table cost outweighs it. */
+ * works through whole tables (a table's hot rows are then fetched into one L2 instead of all
+ * eight).  The table-major work list is cut into eight segments of equal estimated cost;
+ * `table_cost` supplies the estimate (large tables whose rows come from HBM cost more per bag
+ * than small cache-resident ones), without it all tables count the same. */
 #define FWDMI_BAG_XCD_TABLE_AFFINITY 1
 
 /*
@@ -148,6 +152,14 @@ typedef struct fwdmi_bag_table {
 int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_tables, int64_t n_bags,
                               void* output, int32_t dim, int32_t op_type, double avg_bag_len,
                               const fwdmi_bag_ext* ext, void* stream);
+
+/*
+ * Cost estimate for fwdmi_bag_ext.table_cost from the tables' sizes: cost[t] = 1 for a table
+ * small enough to stay in one XCD's L2, growing with log(size) to about 1.45 for a table of
+ * 512 MiB or more, whose rows mostly come from HBM.  (No counterpart in the reference, which
+ * launches one kernel per table.)
+ */
+int fwdmi_bag_table_cost(const int64_t* table_bytes, int32_t n_tables, float* cost);
 
 /*
  * out = gamma * (x - mean) * rsqrt(var + eps) + beta,  x = input (+ bias), per row of ld.

@@ -2,6 +2,8 @@
 import re
 import subprocess
 
+import numpy as np
+
 from forward_amd import lib
 
 
@@ -49,3 +51,13 @@ def test_launchers_validate_before_touching_the_gpu():
     rc = lib.dll.fwdmi_emb_layer_norm(None, 4, 2, 8, None, None, None, None, None, None, None, None, 1, 1, 1, None,
                                       None, lib.F16, 0.0, None)
     assert rc == lib.ERR_BAD_ARG
+
+
+def test_table_cost_estimate():
+    import ctypes as C
+    nbytes = np.array([1 << 10, 2 << 20, 32 << 20, 512 << 20, 8 << 30], np.int64)
+    cost = np.zeros(5, np.float32)
+    assert lib.dll.fwdmi_bag_table_cost(nbytes.ctypes.data, 5, cost.ctypes.data) == 0
+    assert cost[0] == 1.0 and cost[1] == 1.0 and cost[3] == cost[4] and 1.0 < cost[2] < cost[3] < 2.0
+    np.testing.assert_allclose(cost[2], 1.0 + 0.45 * 0.5, rtol=1e-6)    # 32 MiB is half way in log size
+    assert lib.dll.fwdmi_bag_table_cost(None, 5, cost.ctypes.data) == lib.ERR_BAD_ARG

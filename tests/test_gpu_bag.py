@@ -157,6 +157,13 @@ def test_multi_table_concatenated(oracle):
         ops.embedding_bag(batch.tables[t], batch.indices[t], batch.offsets[t], "sum", out=out, out_col=128 * t)
     assert_bits_equal(host(out), want, "per-table launches")
     assert_bits_equal(host(batch.forward(xcd_table_affinity=True)), want, "fused, per-XCD table affinity")
+    # the XCD segmentation may cut the work list anywhere: every bag is still reduced exactly once
+    for cost in ([1, 1, 1, 1, 1], [1e-3, 1, 1e3, 1, 1e-3], [1e6, 1, 1, 1, 1], [1, 1, 1, 1, 1e6], [3, 1, 4, 1, 5]):
+        out = torch.full((3000, 640), 7.0, dtype=torch.float16, device="cuda")
+        batch.forward(out=out, xcd_table_affinity=True, table_cost=np.array(cost, np.float32))
+        assert_bits_equal(host(out), want, "XCD segments for cost %r" % (cost,))
+    with pytest.raises(lib.FwdmiError, match="table_cost"):
+        batch.forward(xcd_table_affinity=True, table_cost=np.array([1, 1, 0, 1, 1], np.float32))
     got32 = host(batch.forward(out_dtype=torch.float32))
     np.testing.assert_allclose(got32, want.astype(np.float32), atol=1e-2, rtol=5e-3)
 

@@ -144,13 +144,31 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   for (int i = tid; i < kLenBuckets; i += wg_lanes) s_hist[i] = 0;
   __syncthreads();
 
+  // A "compact" table has at most 2^24 rows and 4 GiB: a row number fits 32 bits (whatever the
+  // id type) and a row's byte offset is one 24-bit multiply-add on top of a uniform base.
+  // Uniform over the workgroup.
+  const uint32_t row_bytes = (uint32_t)L.dim * (uint32_t)sizeof(TW);
+  const bool compact = T.count <= (1 << 24) && row_bytes < (1u << 24) &&
+                       (uint64_t)T.count * row_bytes <= ((uint64_t)1 << 32);
+  const uint32_t last32 = (uint32_t)(T.count - 1);
+  uint32_t* const s_row = reinterpret_cast<uint32_t*>(s_idx);  // the id window, compact tables
+
   // ---- stage the ids (and weights) the run covers ----------------------------------------
+  // For a compact table the window holds row numbers (id - data_offset; 0xFFFFFFFF for an id
+  // outside the table): the 64-bit part of the range check is done once per id here, not once
+  // per lane that reads the row.
   const int64_t span0 = s_off[0];
   const int64_t span = s_off[nb] - span0;
   const bool staged = span >= 0 && span <= kIdxCap;  // uniform over the workgroup
   if (staged) {
     for (int i = tid; i < span; i += wg_lanes) {
-      s_idx[i] = ids[span0 + i];
+      const TI id = ids[span0 + i];
+      if (compact) {
+        const uint64_t row = (uint64_t)((int64_t)id - T.data_offset);
+        s_row[i] = row < (uint64_t)T.count ? (uint32_t)row : 0xFFFFFFFFu;
+      } else {
+        s_idx[i] = id;
+      }
       if (KIND == kWeighted) s_w[i] = (float)psw[span0 + i];
     }
   }
@@ -200,13 +218,6 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
 
   const TW FWDMI_GLOBAL* __restrict__ tab = gconst<TW>(T.data);
   const int n_units = nb * L.n_slices;
-  // Conditions of the 32-bit ("compact") id / address arithmetic, uniform over the workgroup.
-  const uint32_t row_bytes = (uint32_t)L.dim * (uint32_t)sizeof(TW);
-  const bool compact = sizeof(TI) == 4 && T.data_offset >= 0 && T.data_offset + T.count <= ((int64_t)1 << 31) &&
-                       T.count <= (1 << 24) && row_bytes < (1u << 24) &&
-                       (uint64_t)T.count * row_bytes <= ((uint64_t)1 << 32);
-  const uint32_t lo32 = (uint32_t)T.data_offset;
-  const uint32_t last32 = (uint32_t)(T.count - 1);
   const char FWDMI_GLOBAL* const tab_bytes = gconst<char>(T.data);
   bool oob = false;
   const float one = L.one;
@@ -247,17 +258,23 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
       float w[UU];
       bool ok[UU];
       bool all_ok = true;
+      uint32_t r32[COMPACT ? UU : 1];
       if (LDS) {
         // one LDS address per step; the unrolled reads use immediate offsets
         const uint32_t li = (uint32_t)(i - span0);
         const TI* const sp = s_idx + li;
+        const uint32_t* const rp = s_row + li;
         const float* const wp = s_w + li;
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
           id[u] = 0;
+          if (COMPACT) r32[u] = 0;
           w[u] = 0.0f;
           if (!PRED || u < cnt) {
-            id[u] = sp[u];
+            if (COMPACT)
+              r32[u] = rp[u];
+            else
+              id[u] = sp[u];
             if (KIND == kWeighted) w[u] = wp[u];
           }
         }
@@ -279,7 +296,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
           const bool valid = !PRED || u < cnt;
-          const uint32_t row = valid ? (uint32_t)id[u] - lo32 : 0u;
+          const uint32_t row = r32[u];  // 0 for a row past `cnt`
           worst = max(worst, row);
           const uint32_t off = __umul24(min(row, last32), row_bytes) + col_bytes;
           if (valid) {
@@ -288,7 +305,10 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
 #pragma unroll
             for (int e = 0; e < VEC; ++e) v[u].v[e] = (TW)0.0f;
           }
-          if (KIND == kMax) ok[u] = valid && row <= last32;
+          if (KIND == kMax) {
+            ok[u] = valid && row <= last32;
+            id[u] = (TI)((int64_t)row + T.data_offset);  // argmax reports the id
+          }
         }
         all_ok = worst <= last32;
       } else {
@@ -311,7 +331,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
         oob |= !all_ok;
 #pragma unroll
         for (int u = 0; u < UU; ++u) {
-          if (COMPACT) ok[u] = (!PRED || u < cnt) && ((uint32_t)id[u] - lo32) <= last32;
+          if (COMPACT) ok[u] = (!PRED || u < cnt) && r32[u] <= last32;
           if (!ok[u]) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) v[u].v[e] = (TW)0.0f;

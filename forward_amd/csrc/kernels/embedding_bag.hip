@@ -51,7 +51,8 @@ constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting 
   __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kWeighted || sizeof(TI) == 8) ? 4 : FWDMI_BAG_WAVES_PER_EU)))
 constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 
-enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3 };
+// kMax also tracks the argmax (needs max_indices); kMaxValue is the plugin's case: values only
+enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3, kMaxValue = 4 };
 
 struct BagLaunch {
   const fwdmi_bag_table* tables;  // device array, or nullptr -> `single`
@@ -237,6 +238,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     const bool in_lds = staged && start >= span0 && end <= span0 + span;
 
     float acc[VEC];
+    constexpr bool kIsMax = KIND == kMax || KIND == kMaxValue;
     TI arg[KIND == kMax ? VEC : 1];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
@@ -305,10 +307,8 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
 #pragma unroll
             for (int e = 0; e < VEC; ++e) v[u].v[e] = (TW)0.0f;
           }
-          if (KIND == kMax) {
-            ok[u] = valid && row <= last32;
-            id[u] = (TI)((int64_t)row + T.data_offset);  // argmax reports the id
-          }
+          if (kIsMax) ok[u] = valid && row <= last32;
+          if (KIND == kMax) id[u] = (TI)((int64_t)row + T.data_offset);  // argmax reports the id
         }
         all_ok = worst <= last32;
       } else {
@@ -338,7 +338,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
             w[u] = 0.0f;
           }
         }
-      } else if (COMPACT && KIND != kMax) {
+      } else if (COMPACT && !kIsMax) {
 #pragma unroll
         for (int u = 0; u < UU; ++u) ok[u] = true;
       }
@@ -359,11 +359,11 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
           } else {
             if (ok[u] && (first || x > acc[e])) {
               acc[e] = x;
-              arg[e] = id[u];
+              if (KIND == kMax) arg[e] = id[u];
             }
           }
         }
-        if (KIND == kMax && ok[u]) first = false;
+        if (kIsMax && ok[u]) first = false;
       }
     };
     auto bag = [&](auto lds_tag, auto compact_tag) {
@@ -457,6 +457,9 @@ int launch_kind(int kind, const BagLaunch& L, const BagShape& sh, hipStream_t st
       break;
     case kWeighted:
       hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kWeighted>), grid, block, sh.lds, stream, L);
+      break;
+    case kMaxValue:
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMaxValue>), grid, block, sh.lds, stream, L);
       break;
     default:
       hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMax>), grid, block, sh.lds, stream, L);
@@ -570,7 +573,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                 ((out_stride * so) % store_align) == 0 &&
                 (tables_dev || (single.out_col * so) % store_align == 0);
 
-  const int kind = op == FWDMI_OP_MAX ? kMax : op == FWDMI_OP_SQUARE_SUM ? kSquare : (x.per_sample_weights ? kWeighted : kPlain);
+  const int kind = op == FWDMI_OP_MAX ? (x.max_indices ? kMax : kMaxValue) : op == FWDMI_OP_SQUARE_SUM ? kSquare : (x.per_sample_weights ? kWeighted : kPlain);
   L.psw = x.per_sample_weights;
   int grid = (int)(wgs * n_tables);
   L.total_wgs = grid;

@@ -51,6 +51,42 @@ def test_config2_scaled(oracle, tdt, idt, mode):
         arg = host(res[1])
         assert arg.dtype == idt
         np.testing.assert_array_equal(arg, warg)
+        # the plugin's form: values only (a kernel variant of its own, without the index registers)
+        assert_bits_equal(host(run_bag(wl.table, wl.indices, wl.offsets, m)), want, "max, values only")
+
+
+def test_max_ties_nan_and_empty_bags_match_libtorch_vectors(torch_vectors):
+    """The committed libtorch CPU vectors (first maximum wins, NaN never replaces a value, a NaN
+    first element stays, argmax is the row id, empty bags give 0 / 0) through the HIP path."""
+    v = torch_vectors
+    w, idx, off = v["tie_table"], v["tie_idx"], v["tie_off"]
+    out, arg = run_bag(w, idx, off, "max", want_max_indices=True)
+    assert_bits_equal(host(out), v["tie_max_out"], "max values")
+    np.testing.assert_array_equal(host(arg), v["tie_max_arg"])
+    assert_bits_equal(host(run_bag(w, idx, off, "max")), v["tie_max_out"], "max values, no indices")
+    wq, ridx, roff = v["rnd_tableq"], v["rnd_idx"], v["rnd_off"]
+    for i, o, key in ((ridx, roff, ""), (ridx.astype(np.int32), roff.astype(np.int32), "_i32")):
+        out, arg = run_bag(wq, i, o, "max", want_max_indices=True)
+        assert_bits_equal(host(out), v["rnd_max" + key], "max on the quantised table")
+        np.testing.assert_array_equal(host(arg), v["rnd_max_arg" + key])
+        assert_bits_equal(host(run_bag(wq, i, o, "max")), v["rnd_max" + key], "no indices")
+    assert_bits_equal(host(run_bag(wq.astype(np.float16), ridx, roff, "max")), v["rnd_max_f16"], "fp16 max")
+
+
+@pytest.mark.parametrize("tdt", [np.float32, np.float16])
+def test_max_special_values_against_oracle(oracle, tdt):
+    """Rows full of ties, signed zeros, infinities and NaN in every position of a bag."""
+    rng = np.random.Generator(np.random.PCG64(404))
+    specials = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 0.5, 2.0], np.float32)
+    table = specials[rng.integers(0, specials.size, size=(300, 16))].astype(tdt)
+    lengths = rng.integers(0, 12, size=500)
+    off = np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(np.int32)
+    idx = rng.integers(0, 300, size=int(lengths.sum())).astype(np.int32)
+    want, warg, _ = oracle.embedding_bag(table, idx, off, oracle.OP_MAX, want_max_indices=True)
+    out, arg = run_bag(table, idx, off, "max", want_max_indices=True)
+    assert_bits_equal(host(out), want, "values")
+    np.testing.assert_array_equal(host(arg), warg)
+    assert_bits_equal(host(run_bag(table, idx, off, "max")), want, "values, no indices")
 
 
 def test_config2_full_size_sum_fp16(oracle):

@@ -9,7 +9,9 @@
 //     slices of 64 lanes and a (bag, slice) pair becomes the unit of work.
 //   * A workgroup owns a contiguous run of bags.  Their offsets, and the ids (and weights)
 //     they cover, are copied into LDS once with coalesced loads; slots then read ids from
-//     LDS as broadcasts, so the only per-row global traffic is the row itself.
+//     LDS as broadcasts, so the only per-row global traffic is the row itself.  For tables of
+//     at most 2^24 rows and 4 GiB the copy turns each id (int32 or int64) into a 32-bit row
+//     number, so the 64-bit part of the range check happens once per id.
 //   * The run's bags are ranked by length in LDS and handed out longest first from an LDS
 //     counter: the slots of a wavefront, which execute in lock-step, get bags of nearly equal
 //     length, and the long tail of bag lengths is evened out inside a workgroup.

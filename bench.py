@@ -212,6 +212,10 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
             ms = time_graph(torch, fn2)
             ex["config5_skip_layer_norm"] = {"tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
                                              "algorithmic_GBs": wl.skip_algorithmic_bytes() / (ms * 1e-3) / 1e9}
+            # a yardstick of the same size and traffic (two reads, one write per element): torch's add
+            ms_add = time_graph(torch, lambda: torch.add(x, sk, out=o2))
+            ex["config5_same_traffic_torch_add"] = {"ms": ms_add,
+                                                    "GBs": wl.skip_algorithmic_bytes() / (ms_add * 1e-3) / 1e9}
             # the same two stages in one pass (no intermediate round trip through HBM)
             fn3 = lambda: ops.emb_layer_norm(*a, eps=wl.eps, out=o2, mask_idx=midx, skip=sk, gamma2=g, beta2=b,
                                              bias2=bi, eps2=wl.eps)

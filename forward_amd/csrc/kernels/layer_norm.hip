@@ -58,6 +58,7 @@ struct LnLaunch {
   int32_t total_waves; // row-processing wavefronts in the grid
   float eps;
   float eps2;
+  float one;  // 1.0f, as a run-time value (see the row sum in ln_rows_kernel)
   int32_t batch_major;  // kEmb*: ids / mask are [B,S] and rows are ordered b*S + s
 };
 
@@ -78,7 +79,8 @@ struct Welford {
 __device__ __forceinline__ Welford merge(const Welford a, const Welford b) {
   Welford r;
   r.n = a.n + b.n;
-  const float inv = r.n > 0.0f ? 1.0f / r.n : 0.0f;
+  // counts are small integers: the hardware reciprocal (1 ulp) is ample here
+  const float inv = r.n > 0.0f ? __builtin_amdgcn_rcpf(r.n) : 0.0f;
   const float d = b.mean - a.mean;
   r.mean = a.mean + d * (b.n * inv);
   r.m2 = a.m2 + b.m2 + d * d * (a.n * b.n * inv);
@@ -114,6 +116,35 @@ __device__ __forceinline__ Welford wave_allreduce(Welford w) {
   return w;
 }
 
+// The same when every lane starts with the same count `n0`: the two sides of every merge then
+// hold equal counts, which turns the update into mean = (a + b) / 2 and
+// M2 = M2a + M2b + (b - a)^2 * n / 2 with n known at compile time per level.
+struct MeanM2 {
+  float mean, m2;
+};
+__device__ __forceinline__ MeanM2 merge_equal(const MeanM2 a, const MeanM2 b, float half_n) {
+  const float d = b.mean - a.mean;
+  return MeanM2{__builtin_fmaf(d, 0.5f, a.mean), __builtin_fmaf(d * d, half_n, a.m2 + b.m2)};
+}
+template <int CTRL>
+__device__ __forceinline__ MeanM2 dpp(const MeanM2 w) {
+  return MeanM2{dpp<CTRL>(w.mean), dpp<CTRL>(w.m2)};
+}
+__device__ __forceinline__ Welford wave_allreduce_equal(float mean, float m2, float n0) {
+  MeanM2 w{mean, m2};
+  w = merge_equal(w, dpp<0xB1>(w), 0.5f * n0);
+  w = merge_equal(w, dpp<0x4E>(w), 1.0f * n0);
+  w = merge_equal(w, dpp<0x141>(w), 2.0f * n0);
+  w = merge_equal(w, dpp<0x140>(w), 4.0f * n0);
+  w = merge_equal(w, MeanM2{__shfl_xor(w.mean, 16), __shfl_xor(w.m2, 16)}, 8.0f * n0);
+  w = merge_equal(w, MeanM2{__shfl_xor(w.mean, 32), __shfl_xor(w.m2, 32)}, 16.0f * n0);
+  Welford r;
+  r.n = 64.0f * n0;
+  r.mean = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(w.mean)));
+  r.m2 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(w.m2)));
+  return r;
+}
+
 __device__ __forceinline__ int wave_min(int v) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) v = min(v, __shfl_xor(v, m));
@@ -144,7 +175,8 @@ struct RowRegs {
   bool ok0, ok1, ok2;
 };
 
-template <typename T, int VEC, int NV, int MODE>
+// FULL: ld == 64 * VEC * NV, i.e. every lane owns NV live slices (no masking, equal counts).
+template <typename T, int VEC, int NV, int MODE, bool FULL>
 __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   const int lane = threadIdx.x & 63;
   const int wave_in_wg = threadIdx.x >> 6;
@@ -170,7 +202,7 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int c = (j * 64 + lane) * VEC;
-    live[j] = c < L.ld;
+    live[j] = FULL || c < L.ld;
     col[j] = live[j] ? c : 0;
     if (live[j]) cnt += (float)VEC;
   }
@@ -225,20 +257,32 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   }
 
   bool oob = false;
+  const float one = L.one;
   for (; r < L.rows; r += L.total_waves) {
     // the next row's loads are in flight while this row is reduced
     const int64_t rn = r + L.total_waves;
     if (rn < L.rows) fetch(rn, nxt);
 
     float x[NV][VEC];
-    if (is_emb(MODE)) oob |= !(cur.ok0 && cur.ok1 && cur.ok2);
+    if (is_emb(MODE) && !(cur.ok0 && cur.ok1 && cur.ok2)) {  // uniform and rare: an id outside its table
+      oob = true;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        if (!cur.ok0) cur.a[j] = Pack<T, VEC>{};
+        if (!cur.ok1) cur.b[j] = Pack<T, VEC>{};
+        if (!cur.ok2) cur.c[j] = Pack<T, VEC>{};
+      }
+    }
+    // fma(b, 1, a) rounds exactly like a + b and lets half-precision operands enter the sum
+    // without conversions of their own (mixed-precision FMA); `one` is a kernel argument so that
+    // the multiplication is not folded away.
 #pragma unroll
     for (int j = 0; j < NV; ++j)
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        float v = cur.ok0 ? (float)cur.a[j].v[e] : 0.0f;
-        if (MODE != kLayerNorm) v += cur.ok1 ? (float)cur.b[j].v[e] : 0.0f;
-        if (is_emb(MODE)) v += cur.ok2 ? (float)cur.c[j].v[e] : 0.0f;
+        float v = (float)cur.a[j].v[e];
+        if (MODE != kLayerNorm) v = __builtin_fmaf((float)cur.b[j].v[e], one, v);
+        if (is_emb(MODE)) v = __builtin_fmaf((float)cur.c[j].v[e], one, v);
         x[j][e] = is_emb(MODE) ? v : v + bi[j][e];
       }
 
@@ -248,18 +292,19 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
 #pragma unroll
       for (int j = 0; j < NV; ++j)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) sum += live[j] ? x[j][e] : 0.0f;
+        for (int e = 0; e < VEC; ++e) sum += (FULL || live[j]) ? x[j][e] : 0.0f;
       Welford w{cnt, sum * inv_cnt, 0.0f};
 #pragma unroll
       for (int j = 0; j < NV; ++j)
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          const float d = live[j] ? x[j][e] - w.mean : 0.0f;
+          const float d = (FULL || live[j]) ? x[j][e] - w.mean : 0.0f;
           w.m2 = __builtin_fmaf(d, d, w.m2);
         }
-      w = wave_allreduce(w);
+      w = FULL ? wave_allreduce_equal(w.mean, w.m2, (float)(NV * VEC)) : wave_allreduce(w);
       mu = w.mean;
-      rs = 1.0f / sqrtf(w.m2 / w.n + eps);
+      // hardware reciprocal and reciprocal square root (1 ulp each) instead of the IEEE sequences
+      rs = __builtin_amdgcn_rsqf(__builtin_fmaf(w.m2, __builtin_amdgcn_rcpf(w.n), eps));
     };
     float mu, rs;
     stats(L.eps, mu, rs);
@@ -287,7 +332,7 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           o.v[e] = round_to<T>(__builtin_fmaf(g[j][e], (x[j][e] - mu) * rs, be[j][e]));
-          x[j][e] = (float)o.v[e] + (float)cur.d[j].v[e] + (L.bias2 ? b2.v[e] : 0.0f);
+          x[j][e] = __builtin_fmaf((float)cur.d[j].v[e], one, (float)o.v[e]) + (L.bias2 ? b2.v[e] : 0.0f);
         }
         if (ep && live[j]) gstore<T, VEC>(ep + col[j], o);
       }
@@ -391,14 +436,23 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
 
   const int chunks = (L.ld + 64 * kVec - 1) / (64 * kVec);
   if (vec_ok && (L.ld % kVec) == 0 && chunks <= 8) {
-    if (chunks <= 1)
-      hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 1, MODE>), grid, block, 0, stream, L);
-    else if (chunks <= 2)
-      hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 2, MODE>), grid, block, 0, stream, L);
-    else if (chunks <= 4)
-      hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 4, MODE>), grid, block, 0, stream, L);
-    else
-      hipLaunchKernelGGL((ln_rows_kernel<T, kVec, 8, MODE>), grid, block, 0, stream, L);
+    const int nv = chunks <= 1 ? 1 : chunks <= 2 ? 2 : chunks <= 4 ? 4 : 8;
+    const bool full = L.ld == 64 * kVec * nv;
+#define FWDMI_LN_LAUNCH(NV_)                                                                           \
+  if (full)                                                                                            \
+    hipLaunchKernelGGL((ln_rows_kernel<T, kVec, NV_, MODE, true>), grid, block, 0, stream, L);         \
+  else                                                                                                 \
+    hipLaunchKernelGGL((ln_rows_kernel<T, kVec, NV_, MODE, false>), grid, block, 0, stream, L)
+    if (nv == 1) {
+      FWDMI_LN_LAUNCH(1);
+    } else if (nv == 2) {
+      FWDMI_LN_LAUNCH(2);
+    } else if (nv == 4) {
+      FWDMI_LN_LAUNCH(4);
+    } else {
+      FWDMI_LN_LAUNCH(8);
+    }
+#undef FWDMI_LN_LAUNCH
   } else if constexpr (MODE == kEmbSkip) {
     return set_error(FWDMI_ERR_UNSUPPORTED, "fused emb+skip layer norm needs 16-byte sliceable rows");
   } else {
@@ -437,6 +491,7 @@ int fwdmi_skip_layer_norm(void* stream, int32_t ld, int64_t n, const void* input
   if (n == 0) return FWDMI_OK;
   FWDMI_REQUIRE(input && output && beta && gamma, "layer norm: null pointer");
   LnLaunch L{};
+  L.one = 1.0f;
   L.input = input;
   L.skip = skip;
   L.gamma = gamma;
@@ -475,6 +530,7 @@ int fwdmi_emb_layer_norm_ex(void* stream, int32_t S, int32_t B, int32_t ld, cons
   const bool fused = ext && ext->skip;
   FWDMI_REQUIRE(!fused || (ext->gamma2 && ext->beta2), "emb layer norm: fused stage needs gamma2 and beta2");
   LnLaunch L{};
+  L.one = 1.0f;
   L.input = word;
   L.pos = pos;
   L.tok = tok;

@@ -212,8 +212,13 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   // Issues the loads of row r (no use of the data yet).
   auto fetch = [&](int64_t r, Regs& R) {
     if (is_emb(MODE)) {
-      const int s = L.batch_major ? (int)(r % L.S) : (int)(r / L.B);
-      const int64_t w = ids[r], sg = segs[r];
+      // the row number is the same in every lane; saying so lets the two ids come through the
+      // scalar unit, whose loads return sooner than vector loads
+      const int64_t ru = ((int64_t)__builtin_amdgcn_readfirstlane((int)(r >> 32)) << 32) |
+                         (uint32_t)__builtin_amdgcn_readfirstlane((int)r);
+      const int s = L.batch_major ? (int)(ru % L.S) : (int)(ru / L.B);
+      typedef const int32_t __attribute__((address_space(4))) * ConstIds;  // read-only for the whole launch
+      const int64_t w = ((ConstIds)L.input_ids)[ru], sg = ((ConstIds)L.segment_ids)[ru];
       R.ok0 = w >= 0 && w < L.word_count;
       R.ok1 = s < L.pos_count;
       R.ok2 = sg >= 0 && sg < L.tok_count;

@@ -180,7 +180,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   // the bags its slots hold.  Handing out bags in length order gives the slots of a wavefront
   // bags of (nearly) equal length, and starting with the longest evens out the finish.
   // The order changes which slot reduces a bag, never the result.
-  const bool sorted = L.fixed_len < 0 && nb > 1;
+  const bool sorted = L.fixed_len < 0 && nb > slots;  // with a bag per slot at most there is nothing to order
   if (sorted) {
     // Counting sort on min(length, 255), descending: histogram with LDS atomics, exclusive scan
     // of the 256 buckets by the first wavefront, scatter.  (Order inside a bucket is arbitrary.)

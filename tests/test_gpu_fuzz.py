@@ -1,0 +1,106 @@
+"""Seeded random configurations of the bag reduction through the C ABI against the oracle:
+row width, table / id / output types, mode, weights, offsets form (empty bags, one giant bag,
+include_last_offset), data_offset with ids outside the shard, output column blocks.  Every value
+is compared bit for bit; the out-of-range count must agree with the sticky device flag."""
+import numpy as np
+import pytest
+import torch
+
+from forward_amd import ops
+from gpu_util import assert_bits_equal, dev, host
+
+pytestmark = pytest.mark.gpu
+
+MODES = ("sum", "mean", "max", "square_sum")
+ORACLE_OP = {"sum": 0, "mean": 1, "max": 2, "square_sum": 3}
+
+
+def make_case(seed):
+    r = np.random.Generator(np.random.PCG64(9000 + seed))
+    dim = int(r.choice([1, 3, 8, 16, 24, 32, 64, 96, 128, 200, 256, 520, 1024]))
+    rows = int(r.choice([1, 2, 17, 300, 5000]))
+    tdt = r.choice([np.float32, np.float16])
+    idt = r.choice([np.int32, np.int64])
+    mode = MODES[int(r.integers(0, 4))]
+    weighted = mode == "sum" and r.random() < 0.3
+    n_bags = int(r.choice([1, 2, 5, 33, 200, 1500]))
+    style = int(r.integers(0, 4))
+    if style == 0:      # short bags with many empty ones
+        lengths = r.integers(0, 4, n_bags) * (r.random(n_bags) < 0.6)
+    elif style == 1:    # typical
+        lengths = r.integers(0, 40, n_bags)
+    elif style == 2:    # one bag far longer than the LDS window, the rest tiny
+        lengths = r.integers(0, 3, n_bags)
+        lengths[int(r.integers(0, n_bags))] = int(r.integers(3000, 9000))
+    else:               # all equal
+        lengths = np.full(n_bags, int(r.integers(1, 20)))
+    lengths = lengths.astype(np.int64)
+    n = int(lengths.sum())
+    include_last = bool(r.random() < 0.3)
+    off = np.concatenate([[0], np.cumsum(lengths)])
+    off = (off if include_last else off[:-1]).astype(idt)
+    data_offset = int(r.choice([0, 0, 7, 1000]))
+    spill = r.random() < 0.4                       # some ids outside [data_offset, data_offset + rows)
+    lo, hi = (data_offset - 3, data_offset + rows + 3) if spill else (data_offset, data_offset + rows)
+    idx = r.integers(lo, hi, n).astype(idt)
+    table = (r.standard_normal((rows, dim)) * 0.5).astype(tdt)
+    psw = r.random(n).astype(tdt) if weighted else None
+    odt = tdt if r.random() < 0.7 else (np.float16 if tdt == np.float32 else np.float32)
+    block = bool(r.random() < 0.3) and dim % 8 == 0
+    return dict(table=table, idx=idx, off=off, mode=mode, psw=psw, include_last=include_last,
+                data_offset=data_offset, odt=odt, block=block, n_bags=n_bags, dim=dim, spill=spill)
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_configuration(oracle, seed):
+    c = make_case(seed)
+    want_arg = c["mode"] == "max" and seed % 2 == 0
+    kw = dict(per_sample_weights=c["psw"], include_last_offset=c["include_last"], data_offset=c["data_offset"])
+    tdt = torch.float16 if c["odt"] == np.float16 else torch.float32
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    if c["block"]:
+        width, col = c["dim"] * 3, c["dim"]
+        want = np.full((c["n_bags"], width), 3.0, c["odt"])
+        out = torch.full((c["n_bags"], width), 3.0, dtype=tdt, device="cuda")
+        _, warg, n_oob = oracle.embedding_bag(c["table"], c["idx"], c["off"], ORACLE_OP[c["mode"]], out=want,
+                                              out_col=col, out_dtype=c["odt"], want_max_indices=want_arg, **kw)
+        res = ops.embedding_bag(dev(c["table"]), dev(c["idx"]), dev(c["off"]), c["mode"], out=out, out_col=col,
+                                out_dtype=tdt, want_max_indices=want_arg, oob_flag=flag,
+                                **{**kw, "per_sample_weights": dev(c["psw"])})
+        got = host(out)
+    else:
+        want, warg, n_oob = oracle.embedding_bag(c["table"], c["idx"], c["off"], ORACLE_OP[c["mode"]],
+                                                 out_dtype=c["odt"], want_max_indices=want_arg, **kw)
+        res = ops.embedding_bag(dev(c["table"]), dev(c["idx"]), dev(c["off"]), c["mode"], out_dtype=tdt,
+                                want_max_indices=want_arg, oob_flag=flag,
+                                **{**kw, "per_sample_weights": dev(c["psw"])})
+        got = host(res[0] if want_arg else res)
+    assert_bits_equal(got, want, "seed %d: %s dim %d %s ids, %s table" % (
+        seed, c["mode"], c["dim"], c["idx"].dtype, c["table"].dtype))
+    if want_arg:
+        np.testing.assert_array_equal(host(res[1]), warg)
+    assert bool(flag.item()) == (n_oob > 0)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_fixed_length_and_gather(oracle, seed):
+    r = np.random.Generator(np.random.PCG64(7000 + seed))
+    dim = int(r.choice([1, 4, 16, 64, 100, 128, 384]))
+    rows = int(r.choice([1, 50, 4000]))
+    tdt = r.choice([np.float32, np.float16])
+    idt = r.choice([np.int32, np.int64])
+    b, l = int(r.choice([1, 7, 300, 2000])), int(r.choice([1, 2, 5, 31, 130]))
+    data_offset = int(r.choice([0, 11]))
+    spill = 2 if r.random() < 0.4 else 0
+    ids = r.integers(data_offset - spill, data_offset + rows + spill, (b, l)).astype(idt)
+    table = (r.standard_normal((rows, dim)) * 0.5).astype(tdt)
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    if seed % 3 == 0:
+        want, n_oob = oracle.gather(table, ids, data_offset=data_offset)
+        got = host(ops.gather(dev(table), dev(ids), data_offset=data_offset, oob_flag=flag))
+    else:
+        mode = MODES[int(r.integers(0, 4))]
+        want, _, n_oob = oracle.embedding_bag(table, ids, None, ORACLE_OP[mode], data_offset=data_offset)
+        got = host(ops.embedding_bag_fixed(dev(table), dev(ids), mode, data_offset=data_offset, oob_flag=flag))
+    assert_bits_equal(got.reshape(want.shape), want, "seed %d" % seed)
+    assert bool(flag.item()) == (n_oob > 0)

@@ -187,7 +187,10 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
     }
     return;
   }
-  const int wave = blockIdx.x * kWavesPerWG + wave_in_wg;
+  // The row a wavefront works on is the same in all of its lanes; saying so keeps row addresses
+  // in scalar registers (uniform base + per-lane column offset) and lets the ids of an embedding
+  // row come through the scalar unit.
+  const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * kWavesPerWG + wave_in_wg));
   const T FWDMI_GLOBAL* const in0 = gconst<T>(L.input);
   const T FWDMI_GLOBAL* const in1 = gconst<T>(is_emb(MODE) ? L.pos : L.skip);
   const T FWDMI_GLOBAL* const in3 = gconst<T>(L.skip);
@@ -212,13 +215,9 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   // Issues the loads of row r (no use of the data yet).
   auto fetch = [&](int64_t r, Regs& R) {
     if (is_emb(MODE)) {
-      // the row number is the same in every lane; saying so lets the two ids come through the
-      // scalar unit, whose loads return sooner than vector loads
-      const int64_t ru = ((int64_t)__builtin_amdgcn_readfirstlane((int)(r >> 32)) << 32) |
-                         (uint32_t)__builtin_amdgcn_readfirstlane((int)r);
-      const int s = L.batch_major ? (int)(ru % L.S) : (int)(ru / L.B);
+      const int s = L.batch_major ? (int)(r % L.S) : (int)(r / L.B);
       typedef const int32_t __attribute__((address_space(4))) * ConstIds;  // read-only for the whole launch
-      const int64_t w = ((ConstIds)L.input_ids)[ru], sg = ((ConstIds)L.segment_ids)[ru];
+      const int64_t w = ((ConstIds)L.input_ids)[r], sg = ((ConstIds)L.segment_ids)[r];
       R.ok0 = w >= 0 && w < L.word_count;
       R.ok1 = s < L.pos_count;
       R.ok2 = sg >= 0 && sg < L.tok_count;

@@ -23,8 +23,11 @@
 namespace fwdmi {
 namespace {
 
+// Row-processing workgroups per CU.  With 4 (16 wavefronts per CU) a wavefront of the 8192-token
+// configuration handles two rows, so the second row's loads overlap the first row's arithmetic and
+// store; measured best among 2 / 4 / 6 / 8 / 16.
 #ifndef FWDMI_LN_BLOCKS_PER_CU
-#define FWDMI_LN_BLOCKS_PER_CU 8
+#define FWDMI_LN_BLOCKS_PER_CU 4
 #endif
 constexpr int kWG = 256;
 constexpr int kWavesPerWG = kWG / 64;

@@ -553,7 +553,8 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   if (avg_len < 1.0) avg_len = 1.0;
   // Run length: as many bags as keep the run's ids inside the LDS window, but no more than leaves
   // the chip with ~4 workgroups per CU; small batches also shrink the workgroup (down to one
-  // wavefront) so that every CU gets work.
+  // wavefront) so that every CU gets work, but not below one slot per bag of the run: a slot
+  // that reduces two bags one after the other doubles the launch's critical path.
   const int max_cap = kIdxBytes / (int)dtype_size(x.index_dtype);
   const int64_t total_bags = n_bags * n_tables;
   const int64_t target_wgs = (int64_t)device_cus() * 4;
@@ -561,7 +562,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   const int64_t fit_bags = std::max<int64_t>(1, (int64_t)(max_cap / 1.5 / avg_len));
   want_bags = std::min<int64_t>(std::min(want_bags, fit_bags), kMaxBagsPerWG);
   int block = kWG;
-  while (block > 64 && block / 2 >= lanes && (int64_t)(block / 2 / lanes) * 4 >= want_bags * L.n_slices) block /= 2;
+  while (block > 64 && block / 2 >= lanes && (int64_t)(block / 2 / lanes) >= want_bags * L.n_slices) block /= 2;
   const int slots = block / lanes;
   // a whole number of rounds over the slots
   int64_t units = std::max<int64_t>(slots, want_bags * L.n_slices / slots * slots);

@@ -377,13 +377,87 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
       if (i < end)
         step(std::integral_constant<int, kUnroll - 1>{}, lds_tag, compact_tag, std::true_type{}, i, (int)(end - i));
     };
-    if (in_lds) {
-      if (compact)
-        bag(std::true_type{}, std::true_type{});
-      else
-        bag(std::true_type{}, std::false_type{});
-    } else {
-      bag(std::false_type{}, std::false_type{});
+    // Half-precision maximum without conversions: the running maximum stays packed fp16 (max is
+    // exact in any format) and one packed instruction handles two columns.  Where the packed
+    // maximum could differ from the rule above -- a NaN or an infinity anywhere in the bag's
+    // columns of this lane, a maximum of +-0 (the rule keeps the sign that came first), an id
+    // outside the table -- the lane redoes the bag with the exact loop below; for ordinary data
+    // that never happens.
+    bool exact_needed = true;
+    if constexpr (KIND == kMaxValue && std::is_same<TW, _Float16>::value && VEC == 8) {
+      if (in_lds && compact) {  // uniform over the workgroup, apart from ragged bags
+        typedef _Float16 Half2 __attribute__((ext_vector_type(2)));
+        const Half2 kNegInf = {-__builtin_inff16(), -__builtin_inff16()};
+        const Half2 kZero = {(_Float16)0.0f, (_Float16)0.0f};
+        Half2 m[4] = {kNegInf, kNegInf, kNegInf, kNegInf};
+        Half2 poison[4] = {kZero, kZero, kZero, kZero};  // turns NaN once a NaN or an infinity went by
+        bool bad_id = false;
+        auto fast_step = [&](auto uu_tag, auto pred_tag, int i, int cnt) {
+          constexpr int UU = decltype(uu_tag)::value;
+          constexpr bool PRED = decltype(pred_tag)::value;
+          Pack<TW, VEC> v[UU];
+          uint32_t worst = 0;
+#pragma unroll
+          for (int u = 0; u < UU; ++u) {
+            const bool valid = !PRED || u < cnt;
+            const uint32_t row = valid ? s_row[i + u] : 0u;
+            worst = max(worst, row);
+            const uint32_t off = __umul24(min(row, last32), row_bytes) + col_bytes;
+            if (valid) {
+              v[u] = gload<TW, VEC>(reinterpret_cast<const TW FWDMI_GLOBAL*>(tab_bytes + off));
+            } else {
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) v[u].v[e] = -__builtin_inff16();
+            }
+          }
+          bad_id |= worst > last32;
+#pragma unroll
+          for (int u = 0; u < UU; ++u) {
+            Half2 x[4];
+            __builtin_memcpy(x, &v[u], sizeof(x));
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              // the instruction itself: the generic maximum would first quiet signalling NaNs
+              // of both operands, and NaN is what `poison` already sends to the exact loop
+              asm("v_pk_max_f16 %0, %1, %2" : "=v"(m[k]) : "v"(m[k]), "v"(x[k]));
+              if (!PRED || u < cnt) poison[k] = x[k] * kZero + poison[k];
+            }
+          }
+        };
+        int i = (int)(start - span0);
+        const int stop = (int)(end - span0);
+        for (; i + kUnroll <= stop; i += kUnroll)
+          fast_step(std::integral_constant<int, kUnroll>{}, std::false_type{}, i, kUnroll);
+        if (i < stop) fast_step(std::integral_constant<int, kUnroll - 1>{}, std::true_type{}, i, stop - i);
+        bool doubt = bad_id;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          uint32_t mb, pb;
+          __builtin_memcpy(&mb, &m[k], 4);
+          __builtin_memcpy(&pb, &poison[k], 4);
+          doubt |= (mb & 0x7fffu) == 0 || (mb & 0x7fff0000u) == 0;          // a maximum of +-0
+          doubt |= (pb & 0x7fffu) > 0x7c00u || (pb & 0x7fff0000u) > 0x7c000000u;  // NaN / infinity seen
+        }
+        if (end == start) doubt = false;  // an empty bag is zeros, set below
+        exact_needed = doubt;
+        if (!doubt) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            acc[2 * k] = end > start ? (float)m[k].x : 0.0f;
+            acc[2 * k + 1] = end > start ? (float)m[k].y : 0.0f;
+          }
+        }
+      }
+    }
+    if (exact_needed) {
+      if (in_lds) {
+        if (compact)
+          bag(std::true_type{}, std::true_type{});
+        else
+          bag(std::true_type{}, std::false_type{});
+      } else {
+        bag(std::false_type{}, std::false_type{});
+      }
     }
 
     // ---- epilogue: mean scaling, store ---------------------------------------------------

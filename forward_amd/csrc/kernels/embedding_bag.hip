@@ -449,6 +449,64 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
         }
       }
     }
+    if constexpr (KIND == kMaxValue && std::is_same<TW, float>::value && VEC == 4) {
+      // the same idea for fp32 rows: one v_max_f32 and one poison update per column
+      if (in_lds && compact) {
+        float m[4], poison[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          m[k] = -__builtin_inff();
+          poison[k] = 0.0f;
+        }
+        bool bad_id = false;
+        const float zero = one - one;  // a run-time zero: x * zero must stay a multiplication
+        auto fast_step = [&](auto uu_tag, auto pred_tag, int i, int cnt) {
+          constexpr int UU = decltype(uu_tag)::value;
+          constexpr bool PRED = decltype(pred_tag)::value;
+          Pack<TW, VEC> v[UU];
+          uint32_t worst = 0;
+#pragma unroll
+          for (int u = 0; u < UU; ++u) {
+            const bool valid = !PRED || u < cnt;
+            const uint32_t row = valid ? s_row[i + u] : 0u;
+            worst = max(worst, row);
+            const uint32_t off = __umul24(min(row, last32), row_bytes) + col_bytes;
+            if (valid) {
+              v[u] = gload<TW, VEC>(reinterpret_cast<const TW FWDMI_GLOBAL*>(tab_bytes + off));
+            } else {
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) v[u].v[e] = -__builtin_inff();
+            }
+          }
+          bad_id |= worst > last32;
+#pragma unroll
+          for (int u = 0; u < UU; ++u) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              asm("v_max_f32 %0, %1, %2" : "=v"(m[k]) : "v"(m[k]), "v"(v[u].v[k]));
+              if (!PRED || u < cnt) poison[k] = __builtin_fmaf(v[u].v[k], zero, poison[k]);
+            }
+          }
+        };
+        int i = (int)(start - span0);
+        const int stop = (int)(end - span0);
+        for (; i + kUnroll <= stop; i += kUnroll)
+          fast_step(std::integral_constant<int, kUnroll>{}, std::false_type{}, i, kUnroll);
+        if (i < stop) fast_step(std::integral_constant<int, kUnroll - 1>{}, std::true_type{}, i, stop - i);
+        bool doubt = bad_id;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          doubt |= (__float_as_uint(m[k]) & 0x7fffffffu) == 0;             // a maximum of +-0
+          doubt |= (__float_as_uint(poison[k]) & 0x7fffffffu) > 0x7f800000u;  // NaN / infinity seen
+        }
+        if (end == start) doubt = false;
+        exact_needed = doubt;
+        if (!doubt) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) acc[k] = end > start ? m[k] : 0.0f;
+        }
+      }
+    }
     if (exact_needed) {
       if (in_lds) {
         if (compact)

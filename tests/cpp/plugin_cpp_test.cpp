@@ -8,6 +8,7 @@
 //                          sums computed on the host in double precision
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -95,6 +96,64 @@ int main(int argc, char** argv) {
   CHECK(getPluginRegistry()->getPluginCreator("CustomSkipLayerNormPluginDynamic", "1") != nullptr);
   CHECK(getPluginRegistry()->getPluginCreator("CustomEmbLayerNormPluginDynamic", "1") != nullptr);
   CHECK(getPluginRegistry()->getPluginCreator("EmbeddingBag_TRT", "9") == nullptr);
+
+  // ---- damaged engine bytes: every truncation and a sweep of byte flips of every plugin's blob
+  //      must come back as nullptr or as a plugin that can be destroyed, never as a crash ------
+  {
+    std::vector<float> gamma(16, 1.0f), beta(16, 0.0f), word(5 * 16, 0.25f), pos(4 * 16, 0.5f), tok(2 * 16, 0.125f);
+    const int ld = 16, type_id = FWDMI_F16, fp16 = 1, mha = FWDMI_F16;
+    std::vector<PluginField> ln = {{"ld", &ld, FWDMI_FIELD_I32, 1},           {"type_id", &type_id, FWDMI_FIELD_I32, 1},
+                                   {"beta", beta.data(), FWDMI_FIELD_F32, 16}, {"gamma", gamma.data(), FWDMI_FIELD_F32, 16},
+                                   {"bias", beta.data(), FWDMI_FIELD_F32, 16}};
+    std::vector<PluginField> emb = {{"bert_embeddings_layernorm_beta", beta.data(), FWDMI_FIELD_F32, 16},
+                                    {"bert_embeddings_layernorm_gamma", gamma.data(), FWDMI_FIELD_F32, 16},
+                                    {"bert_embeddings_word_embeddings", word.data(), FWDMI_FIELD_F32, 5 * 16},
+                                    {"bert_embeddings_token_type_embeddings", tok.data(), FWDMI_FIELD_F32, 2 * 16},
+                                    {"bert_embeddings_position_embeddings", pos.data(), FWDMI_FIELD_F32, 4 * 16},
+                                    {"output_fp16", &fp16, FWDMI_FIELD_I32, 1},
+                                    {"mha_type_id", &mha, FWDMI_FIELD_I32, 1}};
+    struct Case {
+      const char* name;
+      const char* version;
+      std::vector<PluginField>* fields;
+    } cases[] = {{"EmbeddingBag_TRT", "001", &field_data},
+                 {"EmbeddingBag_TRT", "002", &field_data},
+                 {"ForwardLayerNormPluginDynamic", "1", &ln},
+                 {"CustomSkipLayerNormPluginDynamic", "1", &ln},
+                 {"CustomEmbLayerNormPluginDynamic", "1", &emb}};
+    for (const Case& c : cases) {
+      IPluginCreator* cr = getPluginRegistry()->getPluginCreator(c.name, c.version);
+      CHECK(cr != nullptr);
+      const PluginFieldCollection fc{(int32_t)c.fields->size(), c.fields->data()};
+      IPluginV2DynamicExt* p = cr->createPlugin("layer", &fc);
+      CHECK(p != nullptr);
+      std::vector<char> good(p->getSerializationSize());
+      p->serialize(good.data());
+      p->destroy();
+      IPluginV2DynamicExt* again = cr->deserializePlugin("layer", good.data(), good.size());
+      CHECK(again != nullptr && again->getSerializationSize() == good.size());
+      again->destroy();
+      for (size_t n = 0; n < good.size(); n += (n < 64 ? 1 : 37)) {
+        std::vector<char> cut(good.begin(), good.begin() + n);  // exact-size heap copy: overreads show up
+        IPluginV2DynamicExt* q = cr->deserializePlugin("layer", cut.data(), cut.size());
+        if (q) q->destroy();
+      }
+      unsigned state = 12345;
+      for (int trial = 0; trial < 400; ++trial) {
+        std::vector<char> bad(good);
+        state = state * 1664525u + 1013904223u;
+        const size_t at = (trial < 200 ? state % std::min<size_t>(bad.size(), 48) : state % bad.size());
+        state = state * 1664525u + 1013904223u;
+        bad[at] = (char)(state >> 24);
+        IPluginV2DynamicExt* q = cr->deserializePlugin("layer", bad.data(), bad.size());
+        if (q) {
+          std::vector<char> out(q->getSerializationSize());
+          q->serialize(out.data());
+          q->destroy();
+        }
+      }
+    }
+  }
 
   // enqueue before configurePlugin is refused with a status
   {

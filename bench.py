@@ -212,10 +212,15 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
             ms = time_graph(torch, fn2)
             ex["config5_skip_layer_norm"] = {"tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
                                              "algorithmic_GBs": wl.skip_algorithmic_bytes() / (ms * 1e-3) / 1e9}
-            # a yardstick of the same size and traffic (two reads, one write per element): torch's add
+            # yardsticks: torch's add on the same tensors (the same traffic, no reduction) and
+            # PyTorch-ROCm's own GPU kernels for the same stage (add + bias, then layer_norm)
             ms_add = time_graph(torch, lambda: torch.add(x, sk, out=o2))
             ex["config5_same_traffic_torch_add"] = {"ms": ms_add,
                                                     "GBs": wl.skip_algorithmic_bytes() / (ms_add * 1e-3) / 1e9}
+            g16, b16, bi16 = g.half(), b.half(), bi.half()
+            H = x.shape[-1]
+            ms_t = time_graph(torch, lambda: torch.nn.functional.layer_norm(x + sk + bi16, (H,), g16, b16, wl.eps))
+            ex["config5_skip_layer_norm_pytorch_rocm_gpu"] = {"ms": ms_t, "tokens_per_s": wl.n_tokens / (ms_t * 1e-3)}
             # the same two stages in one pass (no intermediate round trip through HBM)
             fn3 = lambda: ops.emb_layer_norm(*a, eps=wl.eps, out=o2, mask_idx=midx, skip=sk, gamma2=g, beta2=b,
                                              bias2=bi, eps2=wl.eps)
@@ -232,6 +237,9 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
         ms = time_graph(torch, fn)
         ex["config2_sum_%s_int32" % tname] = {"bags_per_s": wl.n_bags / (ms * 1e-3), "ms": ms,
                                               "algorithmic_GBs": wl.algorithmic_bytes() / (ms * 1e-3) / 1e9}
+        ix64, of64 = ix.long(), of.long()
+        ms_t = time_graph(torch, lambda: torch.nn.functional.embedding_bag(ix64, tb, of64, mode="sum"))
+        ex["config2_sum_%s_pytorch_rocm_gpu" % tname] = {"bags_per_s": wl.n_bags / (ms_t * 1e-3), "ms": ms_t}
     return ex
 
 
@@ -315,6 +323,17 @@ def main():
         cpu["gpu_matches_oracle_on_sample"] = bool(np.array_equal(gpu_out.view(np.uint16), cpu_out.view(np.uint16)))
         result["cpu_baseline"] = cpu
         log("cpu baseline leg %.1fs" % (time.time() - t1))
+    if not args.no_extra and not args.per_table:
+        # the same stage through PyTorch-ROCm's own GPU kernels: 26 embedding_bag launches + cat
+        idx64, off64 = [i.long() for i in idx], [o.long() for o in off]
+        def torch_step():
+            return torch.cat([torch.nn.functional.embedding_bag(idx64[t], tabs[t], off64[t], mode="sum")
+                              for t in range(len(tabs))], dim=1)
+        _, per_t = time_events(torch, torch_step, 5, 2)
+        result["pytorch_rocm_gpu"] = {"ms_per_step": float(np.mean(per_t)),
+                                      "bags_per_s": total_bags / (float(np.mean(per_t)) * 1e-3),
+                                      "what": "26 x torch.nn.functional.embedding_bag (int64 ids) + torch.cat on the same GPU"}
+        del idx64, off64
     if not args.no_extra:
         del tabs, batch
         result["extra"] = extra_measurements(torch, ops, workloads, max(10, args.steps), with_cpu=not args.no_cpu)

@@ -48,9 +48,9 @@ constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting 
 #ifndef FWDMI_BAG_WAVES_PER_EU
 #define FWDMI_BAG_WAVES_PER_EU 6  // register budget of 80 VGPRs: measured best on the 26-table configuration
 #endif
-// max mode, weights and 64-bit ids carry more live registers: they keep the looser budget
+// argmax tracking and weights carry more live registers: they keep the looser budget
 #define FWDMI_BAG_OCCUPANCY \
-  __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kWeighted || sizeof(TI) == 8) ? 4 : FWDMI_BAG_WAVES_PER_EU)))
+  __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kWeighted) ? 4 : FWDMI_BAG_WAVES_PER_EU)))
 constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 
 // kMax also tracks the argmax (needs max_indices); kMaxValue is the plugin's case: values only

@@ -79,7 +79,7 @@ struct BagLaunch {
   int32_t xcd_affinity;      // != 0: XCD x works through work items [xcd_start[x], xcd_start[x+1])
   int32_t xcd_start[kXcds + 1];
   int32_t total_wgs;
-  int32_t idx_cap;    // ids the LDS window holds
+  int32_t idx_cap;    // 32-bit words of the LDS id window: that many row numbers, or half as many 64-bit ids
 };
 
 template <typename TW, typename TI, int VEC, int KIND>
@@ -88,12 +88,11 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
   int64_t* const s_off = reinterpret_cast<int64_t*>(s_raw);
   TI* const s_idx = reinterpret_cast<TI*>(s_off + (L.bags_per_wg + 2));
-  float* const s_w = reinterpret_cast<float*>(s_idx + L.idx_cap);
+  float* const s_w = reinterpret_cast<float*>(reinterpret_cast<uint32_t*>(s_idx) + L.idx_cap);
   int* const s_len = reinterpret_cast<int*>(s_w + (KIND == kWeighted ? L.idx_cap : 0));
   uint16_t* const s_order = reinterpret_cast<uint16_t*>(s_len + L.bags_per_wg);
   __shared__ int s_next;
   __shared__ int s_hist[kLenBuckets];
-  const int kIdxCap = L.idx_cap;
   const int wg_lanes = blockDim.x;
 
   const int tid = threadIdx.x;
@@ -162,7 +161,9 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   // per lane that reads the row.
   const int64_t span0 = s_off[0];
   const int64_t span = s_off[nb] - span0;
-  const bool staged = span >= 0 && span <= kIdxCap;  // uniform over the workgroup
+  // the window holds 32-bit row numbers of a compact table, ids of the launch's type otherwise
+  const int window = compact ? L.idx_cap : L.idx_cap / (int)(sizeof(TI) / 4);
+  const bool staged = span >= 0 && span <= window;  // uniform over the workgroup
   if (staged) {
     for (int i = tid; i < span; i += wg_lanes) {
       const TI id = ids[span0 + i];
@@ -572,8 +573,8 @@ struct BagShape {
 };
 
 // Bytes of the kernel's LDS carve-up.
-size_t bag_lds_bytes(const BagLaunch& L, size_t index_size, bool weighted) {
-  size_t b = (size_t)(L.bags_per_wg + 2) * sizeof(int64_t) + (size_t)L.idx_cap * index_size;
+size_t bag_lds_bytes(const BagLaunch& L, bool weighted) {
+  size_t b = (size_t)(L.bags_per_wg + 2) * sizeof(int64_t) + (size_t)L.idx_cap * sizeof(uint32_t);
   if (weighted) b += (size_t)L.idx_cap * sizeof(float);
   b += (size_t)L.bags_per_wg * (sizeof(int) + sizeof(uint16_t));
   return (b + 15) & ~(size_t)15;
@@ -687,7 +688,14 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   // the chip with ~4 workgroups per CU; small batches also shrink the workgroup (down to one
   // wavefront) so that every CU gets work, but not below one slot per bag of the run: a slot
   // that reduces two bags one after the other doubles the launch's critical path.
-  const int max_cap = kIdxBytes / (int)dtype_size(x.index_dtype);
+  // The id window is sized for 32-bit row numbers unless a single table is known to be too large
+  // for them (more than 2^24 rows or 4 GiB): then it holds the launch's 64-bit ids.  (A multi-table
+  // launch cannot see its tables' sizes here; a run of such a table that does not fit the window
+  // reads its ids from global memory.)
+  const bool i64_ids = x.index_dtype == FWDMI_I64;
+  const bool wide_ids = i64_ids && !tables_dev &&
+                        (single.count > (1 << 24) || (uint64_t)single.count * dim * sw > ((uint64_t)1 << 32));
+  const int max_cap = kIdxBytes / (wide_ids ? 8 : 4);
   const int64_t total_bags = n_bags * n_tables;
   const int64_t target_wgs = (int64_t)device_cus() * 4;
   int64_t want_bags = std::max<int64_t>(1, total_bags / target_wgs);
@@ -699,7 +707,8 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   // a whole number of rounds over the slots
   int64_t units = std::max<int64_t>(slots, want_bags * L.n_slices / slots * slots);
   L.bags_per_wg = (int)std::max<int64_t>(1, std::min<int64_t>(kMaxBagsPerWG, units / L.n_slices));
-  L.idx_cap = std::min(max_cap, std::max(64, next_pow2((int)std::min<double>(max_cap, avg_len * L.bags_per_wg * 2.0))));
+  L.idx_cap = std::min(max_cap, std::max(64, next_pow2((int)std::min<double>(max_cap, avg_len * L.bags_per_wg * 2.0)))) *
+              (wide_ids ? 2 : 1);
   const int64_t wgs = (n_bags + L.bags_per_wg - 1) / L.bags_per_wg;
   FWDMI_REQUIRE(wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
   L.wgs_per_table = (int)wgs;
@@ -746,7 +755,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
     grid = longest * kXcds;
   }
   const bool f16 = x.table_dtype == FWDMI_F16, i64 = x.index_dtype == FWDMI_I64;
-  const BagShape sh{grid, block, bag_lds_bytes(L, dtype_size(x.index_dtype), kind == kWeighted)};
+  const BagShape sh{grid, block, bag_lds_bytes(L, kind == kWeighted)};
   if (f16)
     return i64 ? launch_vec<_Float16, int64_t>(vec, kind, L, sh, stream)
                : launch_vec<_Float16, int32_t>(vec, kind, L, sh, stream);

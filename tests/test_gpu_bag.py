@@ -315,7 +315,26 @@ def test_large_tables_and_offsets_take_the_wide_address_path(oracle):
     sub = host(table[torch.from_numpy(uniq.astype(np.int64)).cuda()])
     want, _, _ = oracle.embedding_bag(sub, inv.astype(np.int32), off, oracle.OP_SUM)
     assert_bits_equal(got, want, "2^24+ rows")
-    del table
+    # the same with int64 ids: the id window then holds 64-bit ids instead of 32-bit row numbers
+    got = host(ops.embedding_bag(table, dev(idx.astype(np.int64)), dev(off.astype(np.int64)), "sum"))
+    assert_bits_equal(got, want, "2^24+ rows, int64 ids")
+    # and inside a multi-table launch, which sizes its runs for row numbers: the large table's
+    # runs do not fit the window as 64-bit ids and read their ids from global memory instead
+    n_bags = 3000
+    lens2 = rng.integers(10, 30, n_bags)
+    off2 = workloads.offsets_from_lengths(lens2, np.int64)
+    idx_big = rng.integers(rows - 5000, rows, int(lens2.sum())).astype(np.int64)
+    small_t = (rng.standard_normal((500, 8)) * 0.25).astype(np.float16)
+    idx_small = rng.integers(0, 500, int(lens2.sum())).astype(np.int64)
+    batch = ops.MultiTableBatch([dev(small_t), table], [dev(idx_small), dev(idx_big)], [dev(off2), dev(off2)])
+    got = host(batch.forward())
+    want_small, _, _ = oracle.embedding_bag(small_t, idx_small, off2, oracle.OP_SUM)
+    uniq, inv = np.unique(idx_big, return_inverse=True)
+    sub = host(table[torch.from_numpy(uniq).cuda()])
+    want_big, _, _ = oracle.embedding_bag(sub, inv.astype(np.int64), off2, oracle.OP_SUM)
+    assert_bits_equal(got[:, :8], want_small, "multi-table, small table")
+    assert_bits_equal(got[:, 8:], want_big, "multi-table, 2^24+ rows with int64 ids")
+    del table, batch
 
     big_rows = 2_200_000                                           # 2.2 M rows x 2 KiB = 4.5 GB > 4 GiB
     big = torch.empty((big_rows, 512), dtype=torch.float32, device="cuda")

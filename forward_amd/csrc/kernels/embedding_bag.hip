@@ -17,6 +17,8 @@
 //     length, and the long tail of bag lengths is evened out inside a workgroup.
 //   * Rows of one bag are added strictly in bag order (eight loads in flight, consumed in
 //     order), so fp32 results do not depend on the launch shape.
+//   * A multi-table launch can give each of the eight XCDs (one L2 each) its own contiguous
+//     part of the table-major work list, cut at equal estimated cost.
 //
 // Memory safety: offsets are clamped to [0, input_size] and made non-decreasing before use,
 // ids outside [data_offset, data_offset+count) never form an address, so arbitrary input
@@ -39,7 +41,7 @@ constexpr int kWG = 256;           // lanes per workgroup (large batches; small 
 #ifndef FWDMI_BAG_IDX_BYTES
 #define FWDMI_BAG_IDX_BYTES 16384
 #endif
-constexpr int kIdxBytes = FWDMI_BAG_IDX_BYTES;   // LDS bytes for staged ids per workgroup (4096 int32 / 2048 int64)
+constexpr int kIdxBytes = FWDMI_BAG_IDX_BYTES;   // LDS bytes of the id window per workgroup (4096 row numbers / 2048 64-bit ids)
 constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
 constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting sort
 #ifndef FWDMI_BAG_UNROLL

@@ -252,9 +252,9 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     bool first = true;
 
     // Loads UU rows starting at bag position i (all loads issued before the first use), then
-    // folds them in bag order.  LDS selects where the ids come from.  COMPACT selects 32-bit
-    // arithmetic: ids are int32, every in-range id is non-negative, the table has at most 2^24
-    // rows and 4 GiB, so a row's byte offset is one 24-bit multiply-add on top of a uniform base.
+    // folds them in bag order.  LDS selects where the ids come from.  COMPACT (implies LDS): the
+    // window holds 32-bit row numbers of a table of at most 2^24 rows and 4 GiB, so a row's byte
+    // offset is one 24-bit multiply-add on top of a uniform base.
     auto step = [&](auto uu_tag, auto lds_tag, auto compact_tag, auto pred_tag, int64_t i, int cnt) {
       constexpr int UU = decltype(uu_tag)::value;
       constexpr bool LDS = decltype(lds_tag)::value;

@@ -28,6 +28,12 @@ def _p(t):
     return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
 
 
+def _require(cond, what):
+    """Argument checks that guard the launchers' memory accesses: raised, never compiled away."""
+    if not cond:
+        raise ValueError("forward_amd.ops: requirement not met: " + what)
+
+
 def _stream(stream):
     s = torch.cuda.current_stream() if stream is None else stream
     return C.c_void_p(s.cuda_stream)
@@ -74,13 +80,14 @@ def embedding_bag(table, indices, offsets, mode="sum", per_sample_weights=None, 
         dst = out
     else:
         _dev(out, "out")
-        assert out.dtype == odt and out.shape[0] == n_bags
+        _require(out.dtype == odt and out.shape[0] == n_bags, 'out.dtype == odt and out.shape[0] == n_bags')
         stride = out.shape[1]
         dst = out.reshape(-1)[out_col:]
     psw = None
     if per_sample_weights is not None:
         psw = _dev(per_sample_weights, "per_sample_weights")
-        assert psw.dtype == table.dtype and psw.numel() == indices.numel()
+        _require(psw.dtype == table.dtype and psw.numel() == indices.numel(),
+                 'psw.dtype == table.dtype and psw.numel() == indices.numel()')
     mi = torch.empty((n_bags, dim), dtype=indices.dtype, device=table.device) if want_max_indices else None
     x = _ext(table, indices, odt, include_last_offset, psw, mi, stride, oob_flag)
     lib.check(lib.dll.fwdmi_embedding_bag(_p(indices), _p(offsets), _p(dst), indices.numel(), n_bags, _p(table),
@@ -92,7 +99,7 @@ def embedding_bag(table, indices, offsets, mode="sum", per_sample_weights=None, 
 def embedding_bag_fixed(table, indices, mode="sum", data_offset=0, out_dtype=None, oob_flag=None, stream=None):
     """Fixed-length bags: ``indices`` is ``[B, L]`` -> ``[B, dim]``."""
     table, indices = _dev(table, "table"), _dev(indices, "indices")
-    assert indices.dim() == 2
+    _require(indices.dim() == 2, 'indices.dim() == 2')
     b, l = indices.shape
     odt = table.dtype if out_dtype is None else out_dtype
     out = torch.empty((b, table.shape[1]), dtype=odt, device=table.device)
@@ -105,7 +112,7 @@ def embedding_bag_fixed(table, indices, mode="sum", data_offset=0, out_dtype=Non
 def gather(table, indices, data_offset=0, out_dtype=None, oob_flag=None, stream=None):
     """Plain row gather: ``[B, L]`` ids -> ``[B, L, dim]``."""
     table, indices = _dev(table, "table"), _dev(indices, "indices")
-    assert indices.dim() == 2
+    _require(indices.dim() == 2, 'indices.dim() == 2')
     b, l = indices.shape
     odt = table.dtype if out_dtype is None else out_dtype
     out = torch.empty((b, l, table.shape[1]), dtype=odt, device=table.device)
@@ -122,7 +129,8 @@ class MultiTableBatch:
     """
 
     def __init__(self, tables, indices, offsets, out_cols=None, data_offsets=None):
-        assert len(tables) == len(indices) == len(offsets) and tables
+        _require(len(tables) == len(indices) == len(offsets) and tables,
+                 'len(tables) == len(indices) == len(offsets) and tables')
         self.tables = [_dev(t, "table") for t in tables]
         self.indices = [_dev(i, "indices") for i in indices]
         self.offsets = [_dev(o, "offsets") for o in offsets]
@@ -133,9 +141,11 @@ class MultiTableBatch:
         data_offsets = [0] * self.n_tables if data_offsets is None else list(data_offsets)
         desc = np.zeros((self.n_tables, 7), np.int64)
         for t in range(self.n_tables):
-            assert self.tables[t].shape[1] == self.dim and self.tables[t].dtype == self.tables[0].dtype
-            assert self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype
-            assert self.offsets[t].numel() == self.n_bags
+            _require(self.tables[t].shape[1] == self.dim and self.tables[t].dtype == self.tables[0].dtype,
+                     'self.tables[t].shape[1] == self.dim and self.tables[t].dtype == self.tables[0].dtype')
+            _require(self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype,
+                     'self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype')
+            _require(self.offsets[t].numel() == self.n_bags, 'self.offsets[t].numel() == self.n_bags')
             desc[t] = (self.tables[t].data_ptr(), self.indices[t].data_ptr(), self.offsets[t].data_ptr(),
                        self.tables[t].shape[0], self.indices[t].numel(), data_offsets[t], out_cols[t])
         self.width = max(out_cols) + self.dim
@@ -155,12 +165,13 @@ class MultiTableBatch:
         if out is None:
             out = torch.empty((self.n_bags, self.width), dtype=odt, device=self.desc.device)
         _dev(out, "out")
-        assert out.dtype == odt and out.shape[0] == self.n_bags and out.shape[1] >= self.width
+        _require(out.dtype == odt and out.shape[0] == self.n_bags and out.shape[1] >= self.width,
+                 'out.dtype == odt and out.shape[0] == self.n_bags and out.shape[1] >= self.width')
         cost = None
         if xcd_table_affinity:
             cost = self.default_table_cost() if table_cost is None else table_cost
             cost = np.ascontiguousarray(cost, np.float32)
-            assert cost.shape == (self.n_tables,)
+            _require(cost.shape == (self.n_tables,), 'cost.shape == (self.n_tables,)')
         x = _ext(self.tables[0], self.indices[0], odt, out_row_stride=out.shape[1], oob_flag=oob_flag,
                  flags=lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0, table_cost=cost)
         avg = self.total_indices / max(1, self.n_bags * self.n_tables)
@@ -171,9 +182,10 @@ class MultiTableBatch:
 
 def _params(gamma, beta, bias=None):
     g, b = _dev(gamma, "gamma"), _dev(beta, "beta")
-    assert g.dtype == torch.float32 and b.dtype == torch.float32
+    _require(g.dtype == torch.float32 and b.dtype == torch.float32,
+             'g.dtype == torch.float32 and b.dtype == torch.float32')
     if bias is not None:
-        assert _dev(bias, "bias").dtype == torch.float32
+        _require(_dev(bias, "bias").dtype == torch.float32, '_dev(bias, "bias").dtype == torch.float32')
     return g, b, bias
 
 
@@ -182,9 +194,10 @@ def skip_layer_norm(x, gamma, beta, skip=None, bias=None, eps=0.0, out=None, str
     x = _dev(x, "input")
     g, b, bias = _params(gamma, beta, bias)
     ld = x.shape[-1]
-    assert g.numel() == ld and b.numel() == ld
+    _require(g.numel() == ld and b.numel() == ld, 'g.numel() == ld and b.numel() == ld')
     if skip is not None:
-        assert _dev(skip, "skip").shape == x.shape and skip.dtype == x.dtype
+        _require(_dev(skip, "skip").shape == x.shape and skip.dtype == x.dtype,
+                 '_dev(skip, "skip").shape == x.shape and skip.dtype == x.dtype')
     out = torch.empty_like(x) if out is None else _dev(out, "out")
     lib.check(lib.dll.fwdmi_skip_layer_norm(_stream(stream), ld, x.numel(), _p(x), _p(skip), _p(b), _p(g), _p(out),
                                             _p(bias), _FDT[x.dtype], eps))
@@ -212,9 +225,10 @@ def emb_layer_norm(input_ids, segment_ids, input_mask, word, pos, tok, gamma, be
     """
     ids, seg = _dev(input_ids, "input_ids"), _dev(segment_ids, "segment_ids")
     msk = _dev(input_mask, "input_mask") if input_mask is not None else None
-    assert ids.dtype == torch.int32 and seg.dtype == torch.int32 and ids.dim() == 2 and seg.shape == ids.shape
+    _require(ids.dtype == torch.int32 and seg.dtype == torch.int32 and ids.dim() == 2 and seg.shape == ids.shape,
+             'ids.dtype == torch.int32 and seg.dtype == torch.int32 and ids.dim() == 2 and seg.shape == ids.shape')
     word, pos, tok = _dev(word, "word"), _dev(pos, "pos"), _dev(tok, "tok")
-    assert word.dtype == pos.dtype == tok.dtype
+    _require(word.dtype == pos.dtype == tok.dtype, 'word.dtype == pos.dtype == tok.dtype')
     g, b, _ = _params(gamma, beta)
     s, bsz = (ids.shape[1], ids.shape[0]) if batch_major else ids.shape
     ld = word.shape[1]
@@ -227,9 +241,11 @@ def emb_layer_norm(input_ids, segment_ids, input_mask, word, pos, tok, gamma, be
     keep = []
     if skip is not None:
         g2, b2, bias2 = _params(gamma2, beta2, bias2)
-        assert _dev(skip, "skip").dtype == word.dtype and skip.numel() == ids.numel() * ld
+        _require(_dev(skip, "skip").dtype == word.dtype and skip.numel() == ids.numel() * ld,
+                 '_dev(skip, "skip").dtype == word.dtype and skip.numel() == ids.numel() * ld')
         if emb_out is not None:
-            assert _dev(emb_out, "emb_out").dtype == word.dtype and emb_out.numel() == skip.numel()
+            _require(_dev(emb_out, "emb_out").dtype == word.dtype and emb_out.numel() == skip.numel(),
+                     '_dev(emb_out, "emb_out").dtype == word.dtype and emb_out.numel() == skip.numel()')
         x.skip, x.gamma2, x.beta2 = skip.data_ptr(), g2.data_ptr(), b2.data_ptr()
         x.bias2 = bias2.data_ptr() if bias2 is not None else None
         x.emb_output = emb_out.data_ptr() if emb_out is not None else None

@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--cpu-bags", type=int, default=4096, help="bags per table in the CPU baseline sample")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device-to-device copy (known traffic, to scale rocprof byte counters)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the benchmark: single-table bag reduction over row widths, table types and "
+                         "bag lengths with uniform random ids, beside torch's GPU embedding_bag (a table on stdout)")
     return ap.parse_args()
 
 
@@ -250,6 +253,35 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
     return ex
 
 
+def sweep(torch, ops):
+    """Regime table of the single-table launcher: 65536 fixed-length bags (8192 for the widest
+    cases) of uniform random int32 ids over a table of up to 1 M rows / 1 GiB; algorithmic bytes
+    per launch as in the benchmark; every case beside torch.nn.functional.embedding_bag on the
+    same GPU, both timed as 10 launches captured in one HIP graph."""
+    import torch.nn.functional as F
+    r = np.random.Generator(np.random.PCG64(5))
+    print("%5s %5s %4s %6s | %9s %9s | %9s | %s" % ("dim", "type", "L", "mode", "ms", "GB/s", "torch ms", "speedup"),
+          flush=True)
+    for tdt in (torch.float16, torch.float32):
+        for dim in (8, 16, 32, 64, 128, 256, 512, 1024):
+            rows = min(1_000_000, (1 << 30) // (dim * 4))
+            table = (torch.randn((rows, dim), device="cuda") * 0.1).to(tdt)
+            sz = table.element_size()
+            for bag_len in (1, 4, 16, 64):
+                nb = 65536 if dim * bag_len <= 128 * 64 else 8192
+                for mode in ("sum", "max") if bag_len == 16 else ("sum",):
+                    idx = torch.from_numpy(r.integers(0, rows, nb * bag_len).astype(np.int32)).cuda()
+                    off = torch.arange(0, nb * bag_len, bag_len, dtype=torch.int32, device="cuda")
+                    out = torch.empty((nb, dim), dtype=tdt, device="cuda")
+                    ms = time_graph(torch, lambda: ops.embedding_bag(table, idx, off, mode, out=out), inner=10, reps=7)
+                    nbytes = nb * bag_len * (dim * sz + 4) + nb * 4 + nb * dim * sz
+                    i64, o64 = idx.long(), off.long()
+                    tms = time_graph(torch, lambda: F.embedding_bag(i64, table, o64, mode=mode), inner=10, reps=5)
+                    print("%5d %5s %4d %6s | %9.4f %9.0f | %9.4f | %.2f" % (
+                        dim, "f16" if sz == 2 else "f32", bag_len, mode, ms, nbytes / ms / 1e6, tms, tms / ms),
+                        flush=True)
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -261,6 +293,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU: the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(1)
+    if args.sweep:
+        sweep(torch, ops)
+        return
 
     t0 = time.time()
     wl = workloads.config4(n_tables=args.tables, n_bags=args.bags)

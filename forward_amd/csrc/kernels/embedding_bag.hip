@@ -643,8 +643,9 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                      x.table_dtype, x.index_dtype, x.out_dtype);
   if (op != FWDMI_OP_SUM && op != FWDMI_OP_MEAN && op != FWDMI_OP_MAX && op != FWDMI_OP_SQUARE_SUM)
     return set_error(FWDMI_ERR_UNSUPPORTED, "embedding bag: unknown op %d", op);
-  FWDMI_REQUIRE(n_bags >= 0 && dim > 0 && n_tables > 0, "embedding bag: n_bags=%lld dim=%d n_tables=%d",
-                (long long)n_bags, dim, n_tables);
+  // dim: a row's byte size and a run's (bag, slice) count stay far inside 32 bits
+  FWDMI_REQUIRE(n_bags >= 0 && dim > 0 && dim <= (1 << 24) && n_tables > 0,
+                "embedding bag: n_bags=%lld dim=%d (1 .. 2^24) n_tables=%d", (long long)n_bags, dim, n_tables);
   FWDMI_REQUIRE(!x.per_sample_weights || op == FWDMI_OP_SUM,
                 "embedding bag: per_sample_weights needs op SUM (got %d)", op);
   FWDMI_REQUIRE(!x.max_indices || (op == FWDMI_OP_MAX && !tables_dev),
@@ -754,6 +755,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
       L.xcd_start[k] = cut;
       longest = std::max(longest, cut - L.xcd_start[k - 1]);
     }
+    FWDMI_REQUIRE((int64_t)longest * kXcds < (int64_t)1 << 31, "embedding bag: grid too large");
     grid = longest * kXcds;
   }
   const bool f16 = x.table_dtype == FWDMI_F16, i64 = x.index_dtype == FWDMI_I64;
@@ -782,7 +784,7 @@ int fwdmi_embedding_bag(const void* input, const void* input_2, void* output, in
 int fwdmi_embedding_bag_fixed(const void* input, void* output, int64_t batch_size, int64_t offset,
                               const void* data, int64_t count, int32_t dim, int64_t data_offset,
                               int32_t op_type, const fwdmi_bag_ext* ext, void* stream) {
-  if (offset < 0 || batch_size < 0)
+  if (offset < 0 || batch_size < 0 || (offset > 0 && batch_size > INT64_MAX / offset))
     return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "fixed-length bags: batch %lld x length %lld",
                             (long long)batch_size, (long long)offset);
   fwdmi_bag_table t{data, input, nullptr, count, batch_size * offset, data_offset, 0};
@@ -792,7 +794,7 @@ int fwdmi_embedding_bag_fixed(const void* input, void* output, int64_t batch_siz
 
 int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t offset, const void* data,
                  int64_t count, int32_t dim, int64_t data_offset, const fwdmi_bag_ext* ext, void* stream) {
-  if (offset < 0 || batch_size < 0)
+  if (offset < 0 || batch_size < 0 || (offset > 0 && batch_size > INT64_MAX / offset))
     return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "gather: batch %lld x %lld", (long long)batch_size,
                             (long long)offset);
   // A gather is a sum over bags of exactly one id.

@@ -44,6 +44,12 @@ def test_launchers_validate_before_touching_the_gpu():
     assert rc == lib.ERR_BAD_ARG                       # null output
     rc = lib.dll.fwdmi_embedding_bag(None, None, None, 0, 0, None, 10, 8, 0, 0, None, None)
     assert rc == lib.OK                                # zero bags: nothing to do
+    rc = lib.dll.fwdmi_embedding_bag(None, None, None, 0, 4, None, 10, (1 << 24) + 1, 0, 0, None, None)
+    assert rc == lib.ERR_BAD_ARG and "dim" in lib.last_error()
+    rc = lib.dll.fwdmi_embedding_bag_fixed(None, None, 1 << 40, 1 << 40, None, 10, 8, 0, 0, None, None)
+    assert rc == lib.ERR_BAD_ARG                       # batch x length leaves 64 bits
+    rc = lib.dll.fwdmi_gather(None, None, 1 << 62, 4, None, 10, 8, 0, None, None)
+    assert rc == lib.ERR_BAD_ARG
     rc = lib.dll.fwdmi_layer_norm(None, 10, 25, None, None, None, None, None, lib.F32, 0.0)
     assert rc == lib.ERR_BAD_ARG and "multiple" in lib.last_error()
     rc = lib.dll.fwdmi_layer_norm(None, 10, 20, None, None, None, None, None, lib.I8, 0.0)

@@ -569,6 +569,19 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   if (oob && L.oob_flag) atomicOr(L.oob_flag, 1);
 }
 
+// Descriptors of a multi-table batch travel to device memory as kernel arguments: no staging
+// buffer on the host, no copy engine, ordered on the stream like any launch.
+constexpr int kFillChunk = 64;  // 64 x 56 bytes of descriptors per launch, inside the 4 KiB argument limit
+struct TableChunk {
+  fwdmi_bag_table t[kFillChunk];
+};
+
+__global__ __launch_bounds__(kFillChunk) void bag_tables_fill_kernel(const TableChunk c, int n,
+                                                                     fwdmi_bag_table* dst) {
+  const int i = threadIdx.x;
+  if (i < n) dst[i] = c.t[i];
+}
+
 struct BagShape {
   int grid, block;
   size_t lds;
@@ -817,6 +830,22 @@ int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_table
   fwdmi_bag_table none{};
   return fwdmi::bag_dispatch(tables_dev, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, ext,
                              static_cast<hipStream_t>(stream));
+}
+
+int fwdmi_bag_tables_fill(const fwdmi_bag_table* tables_host, int32_t n_tables, fwdmi_bag_table* tables_dev,
+                          void* stream) {
+  fwdmi::clear_error();
+  if (n_tables < 0 || (n_tables > 0 && (!tables_host || !tables_dev)))
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "table descriptors: null argument");
+  for (int32_t at = 0; at < n_tables; at += fwdmi::kFillChunk) {
+    const int n = std::min<int32_t>(fwdmi::kFillChunk, n_tables - at);
+    fwdmi::TableChunk c{};
+    std::copy(tables_host + at, tables_host + at + n, c.t);
+    hipLaunchKernelGGL(fwdmi::bag_tables_fill_kernel, dim3(1), dim3(fwdmi::kFillChunk), 0,
+                       static_cast<hipStream_t>(stream), c, n, tables_dev + at);
+    FWDMI_HIP_CHECK(hipGetLastError());
+  }
+  return FWDMI_OK;
 }
 
 // Measured on the 26-table configuration (tables of 0.25 MB .. 2.5 GB): per-bag cost ratios

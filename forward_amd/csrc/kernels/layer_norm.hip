@@ -198,8 +198,6 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   const T FWDMI_GLOBAL* const in1 = gconst<T>(is_emb(MODE) ? L.pos : L.skip);
   const T FWDMI_GLOBAL* const in3 = gconst<T>(L.skip);
   const T FWDMI_GLOBAL* const in2 = gconst<T>(L.tok);
-  const int32_t FWDMI_GLOBAL* const ids = gconst<int32_t>(L.input_ids);
-  const int32_t FWDMI_GLOBAL* const segs = gconst<int32_t>(L.segment_ids);
 
   // Per-lane column slices: chunk j covers elements (j*64 + lane)*VEC .. +VEC.
   bool live[NV];

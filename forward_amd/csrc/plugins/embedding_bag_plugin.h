@@ -11,6 +11,7 @@
 
 #include <memory>
 #include <string>
+#include <vector>
 
 #include "plugin_util.h"
 
@@ -96,6 +97,83 @@ class EmbeddingBagPluginCreator : public BaseCreator {
 class EmbeddingBagPluginCreatorExt : public EmbeddingBagPluginCreator {
  public:
   EmbeddingBagPluginCreatorExt() : EmbeddingBagPluginCreator(true) {}
+};
+
+// ---- all tables of a sparse stage as one plugin --------------------------------------------------
+// "EmbeddingBagGroup_TRT" / "001": T tables of one dim reduce the same number of bags in ONE
+// launch and write the concatenated [B, T*dim] matrix directly.  It stands for the T
+// EmbeddingBag_TRT layers plus the concatenation layer a DLRM-style graph holds (the reference
+// builds one plugin layer per aten::embedding_bag node, layer_creators/trt_embedding_bag_creator.h:44-85,
+// and concatenates afterwards).  Inputs: ids_0 [N_0], offsets_0 [B] or [1, B], ids_1, offsets_1, ...
+// Output t*dim .. (t+1)*dim-1 of every row equals what EmbeddingBag_TRT "002" gives for table t.
+constexpr const char* EMBEDDING_BAG_GROUP_PLUGIN_NAME{"EmbeddingBagGroup_TRT"};
+constexpr const char* EMBEDDING_BAG_GROUP_PLUGIN_VERSION{"001"};
+constexpr int kMaxGroupTables = 1024;
+
+struct EmbeddingBagGroupSpec {
+  int dim = 0;
+  ReduceOperation op = ReduceOperation::SUM;
+  std::vector<int> count;     // rows per table
+  std::vector<int> offset;    // data_offset per table
+  std::vector<float> cost;    // relative cost of one bag per table (balances the per-XCD split)
+  EmbeddingBagOptions opt;    // per_sample_weights is not available in a group
+  int xcd_affinity = 1;
+  int n_tables() const { return (int)count.size(); }
+  size_t total_rows() const {
+    size_t n = 0;
+    for (int c : count) n += (size_t)c;
+    return n;
+  }
+};
+
+class EmbeddingBagGroupPlugin final : public IPluginV2DynamicExt {
+ public:
+  // `tables`: the T tables back to back, table t at row sum(count[0..t)).
+  EmbeddingBagGroupPlugin(std::shared_ptr<HostDeviceBlob> tables, EmbeddingBagGroupSpec spec);
+  static EmbeddingBagGroupPlugin* deserialize(const void* data, size_t length);
+  ~EmbeddingBagGroupPlugin() noexcept override;
+
+  int getNbOutputs() const noexcept override;
+  Dims getOutputDimensions(int outputIndex, const Dims* inputs, int nbInputs) noexcept override;
+  bool supportsFormatCombination(int pos, const PluginTensorDesc* inOut, int nbInputs,
+                                 int nbOutputs) noexcept override;
+  int configurePlugin(const DynamicPluginTensorDesc* in, int nbInputs, const DynamicPluginTensorDesc* out,
+                      int nbOutputs) noexcept override;
+  // Device memory for the T table descriptors of one enqueue.
+  size_t getWorkspaceSize(const PluginTensorDesc* inputs, int nbInputs, const PluginTensorDesc* outputs,
+                          int nbOutputs) const noexcept override;
+  int initialize() noexcept override;
+  void terminate() noexcept override;
+  int enqueue(const PluginTensorDesc* inputDesc, const PluginTensorDesc* outputDesc, const void* const* inputs,
+              void* const* outputs, void* workspace, void* hipStream) noexcept override;
+  size_t getSerializationSize() const noexcept override;
+  void serialize(void* buffer) const noexcept override;
+  const char* getPluginType() const noexcept override;
+  const char* getPluginVersion() const noexcept override;
+  void destroy() noexcept override;
+  IPluginV2DynamicExt* clone() const noexcept override;
+  void setPluginNamespace(const char* pluginNamespace) noexcept override;
+  const char* getPluginNamespace() const noexcept override;
+  DataType getOutputDataType(int index, const DataType* inputTypes, int nbInputs) const noexcept override;
+  int32_t* oobFlagDevice() const noexcept override { return d_oob_; }
+
+ private:
+  EmbeddingBagGroupSpec spec_;
+  std::shared_ptr<HostDeviceBlob> tables_;  // shared with clones
+  void* d_data_ = nullptr;
+  int32_t* d_oob_ = nullptr;
+  bool initialized_ = false;
+  std::string namespace_;
+};
+
+class EmbeddingBagGroupPluginCreator : public BaseCreator {
+ public:
+  EmbeddingBagGroupPluginCreator();
+  const char* getPluginName() const noexcept override;
+  const char* getPluginVersion() const noexcept override;
+  IPluginV2DynamicExt* createPlugin(const char* name, const PluginFieldCollection* fc) noexcept override;
+  IPluginV2DynamicExt* deserializePlugin(const char* name, const void* serialData,
+                                         size_t serialLength) noexcept override;
 };
 
 }  // namespace fwdmi

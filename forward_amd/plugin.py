@@ -99,22 +99,32 @@ class Plugin:
     def terminate(self):
         lib.dll.fwdmi_plugin_terminate(self._h)
 
-    def enqueue_raw(self, in_descs, out_descs, in_ptrs, out_ptrs, stream_handle=None):
+    def enqueue_raw(self, in_descs, out_descs, in_ptrs, out_ptrs, stream_handle=None, workspace_ptr=None):
         """``enqueue`` on raw device addresses; returns the status instead of raising."""
         ins = (C.c_void_p * max(1, len(in_ptrs)))(*in_ptrs)
         outs = (C.c_void_p * max(1, len(out_ptrs)))(*out_ptrs)
         s = torch.cuda.current_stream().cuda_stream if stream_handle is None else stream_handle
-        return lib.dll.fwdmi_plugin_enqueue(self._h, _descs(in_descs), _descs(out_descs), ins, outs, None,
-                                            C.c_void_p(s))
+        return lib.dll.fwdmi_plugin_enqueue(self._h, _descs(in_descs), _descs(out_descs), ins, outs,
+                                            C.c_void_p(workspace_ptr) if workspace_ptr else None, C.c_void_p(s))
 
-    def enqueue(self, inputs, outputs, stream=None):
-        """Device tensors in, device tensors out (written in place); raises on a non-zero status."""
+    def enqueue(self, inputs, outputs, stream=None, workspace=None):
+        """Device tensors in, device tensors out (written in place); raises on a non-zero status.
+        ``workspace``: a device byte tensor of at least ``getWorkspaceSize`` bytes; when the plugin
+        asks for one and none is given, one is allocated (and kept) here, as the engine hosting
+        the plugin would."""
         for t in list(inputs) + list(outputs):
             if not t.is_cuda or not t.is_contiguous():
                 raise RuntimeError("enqueue needs contiguous device tensors")
         s = None if stream is None else stream.cuda_stream
-        rc = self.enqueue_raw([_desc_of(t) for t in inputs], [_desc_of(t) for t in outputs],
-                              [t.data_ptr() for t in inputs], [t.data_ptr() for t in outputs], s)
+        ind, outd = [_desc_of(t) for t in inputs], [_desc_of(t) for t in outputs]
+        if workspace is None:
+            need = self.getWorkspaceSize(ind, outd)
+            if need:
+                if getattr(self, "_ws", None) is None or self._ws.numel() < need:
+                    self._ws = torch.empty(need, dtype=torch.uint8, device=inputs[0].device)
+                workspace = self._ws
+        rc = self.enqueue_raw(ind, outd, [t.data_ptr() for t in inputs], [t.data_ptr() for t in outputs], s,
+                              None if workspace is None else workspace.data_ptr())
         return lib.check(rc)
 
     def __call__(self, *inputs):

@@ -154,6 +154,17 @@ int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_table
                               const fwdmi_bag_ext* ext, void* stream);
 
 /*
+ * Writes n_tables descriptors from HOST memory into the DEVICE array a later
+ * fwdmi_embedding_bag_multi on the same stream reads.  The descriptors travel as kernel
+ * arguments: stream-ordered, no host synchronisation, no pinned staging buffer, and the host
+ * array may be reused as soon as the call returns.  For callers whose id / offset buffers change
+ * from call to call (a plugin's enqueue).  (No counterpart in the reference, which launches one
+ * kernel per table.)
+ */
+int fwdmi_bag_tables_fill(const fwdmi_bag_table* tables_host, int32_t n_tables, fwdmi_bag_table* tables_dev,
+                          void* stream);
+
+/*
  * Cost estimate for fwdmi_bag_ext.table_cost from the tables' sizes: cost[t] = 1 for a table
  * small enough to stay in one XCD's L2, growing with log(size) to about 1.45 for a table of
  * 512 MiB or more, whose rows mostly come from HBM.  (No counterpart in the reference, which

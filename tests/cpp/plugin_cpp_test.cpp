@@ -112,11 +112,18 @@ int main(int argc, char** argv) {
                                     {"bert_embeddings_position_embeddings", pos.data(), FWDMI_FIELD_F32, 4 * 16},
                                     {"output_fp16", &fp16, FWDMI_FIELD_I32, 1},
                                     {"mha_type_id", &mha, FWDMI_FIELD_I32, 1}};
+    const int g_dim = 4, g_op = 0, g_counts[3] = {2, 5, 1};
+    std::vector<float> g_rows(8 * 4, 0.5f);
+    std::vector<PluginField> group = {{"dim", &g_dim, FWDMI_FIELD_I32, 1},
+                                      {"op", &g_op, FWDMI_FIELD_I32, 1},
+                                      {"count", g_counts, FWDMI_FIELD_I32, 3},
+                                      {"data", g_rows.data(), FWDMI_FIELD_F32, 8 * 4}};
     struct Case {
       const char* name;
       const char* version;
       std::vector<PluginField>* fields;
     } cases[] = {{"EmbeddingBag_TRT", "001", &field_data},
+                 {"EmbeddingBagGroup_TRT", "001", &group},
                  {"EmbeddingBag_TRT", "002", &field_data},
                  {"ForwardLayerNormPluginDynamic", "1", &ln},
                  {"CustomSkipLayerNormPluginDynamic", "1", &ln},

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
 def test_basic_calls_without_gpu():
     assert lib.dll.fwdmi_version().startswith(b"fwdmi")
     assert lib.dll.fwdmi_device_count() >= 0
-    assert lib.dll.fwdmi_registry_size() == 5
+    assert lib.dll.fwdmi_registry_size() == 6
 
 
 def test_launchers_validate_before_touching_the_gpu():

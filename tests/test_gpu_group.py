@@ -1,0 +1,156 @@
+"""EmbeddingBagGroup_TRT: the T EmbeddingBag layers + concatenation of a DLRM-style sparse stage as
+one plugin.  Its output must equal, bit for bit, the column blocks that T EmbeddingBag_TRT "002"
+plugins produce one by one, and the oracle's."""
+import numpy as np
+import pytest
+import torch
+
+from forward_amd import lib, plugin, workloads
+from forward_amd.plugin import PluginFieldData as F
+from gpu_util import assert_bits_equal, dev, host
+
+pytestmark = pytest.mark.gpu
+REG = plugin.getPluginRegistry()
+GROUP = REG.getPluginCreator("EmbeddingBagGroup_TRT", "001")
+SINGLE = REG.getPluginCreator("EmbeddingBag_TRT", "002")
+
+
+def group_fields(tables, op=0, extra=()):
+    return [F("dim", tables[0].shape[1]), F("op", op), F("count", np.array([t.shape[0] for t in tables], np.int32)),
+            F("data", np.concatenate([t.reshape(-1) for t in tables]))] + list(extra)
+
+
+def interleave(ids, offs):
+    return [x for pair in zip(ids, offs) for x in pair]
+
+
+def random_batch(rng, rows, n_bags, idt, max_len=12, lo_spill=0):
+    ids, offs = [], []
+    for r in rows:
+        lengths = rng.integers(0, max_len, n_bags)
+        offs.append(np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(idt))
+        ids.append(rng.integers(-lo_spill, r + lo_spill, int(lengths.sum())).astype(idt))
+    return ids, offs
+
+
+@pytest.mark.parametrize("op", [0, 1, 2, 3])
+@pytest.mark.parametrize("tdt,idt,out16", [(np.float16, np.int32, 1), (np.float32, np.int64, 0), (np.float16, np.int64, 0)])
+def test_group_equals_single_table_plugins_and_oracle(oracle, op, tdt, idt, out16):
+    rng = np.random.Generator(np.random.PCG64(400 + op))
+    rows, dim, n_bags = [50, 4000, 7, 900, 20000], 64, 700
+    tables = [(rng.standard_normal((r, dim)) * 0.3).astype(tdt) for r in rows]
+    ids, offs = random_batch(rng, rows, n_bags, idt)
+    it = lib.I64 if idt == np.int64 else lib.I32
+    extra = [F("index_type", it), F("output_fp16", out16)]
+    g = GROUP.createPlugin("sparse", group_fields(tables, op, extra))
+    got = host(g(*[dev(x) for x in interleave(ids, offs)]))
+    odt = np.float16 if out16 else np.float32
+    assert got.shape == (n_bags, len(rows) * dim) and got.dtype == odt
+    for t, tab in enumerate(tables):
+        one = SINGLE.createPlugin("bag", [F("dim", dim), F("count", rows[t]), F("offset", 0), F("op", op),
+                                          F("data", tab)] + extra)
+        block = host(one(dev(ids[t]), dev(offs[t])))
+        assert_bits_equal(got[:, t * dim:(t + 1) * dim], block, "table %d against EmbeddingBag_TRT 002" % t)
+        want, _, _ = oracle.embedding_bag(tab, ids[t], offs[t], op, out_dtype=odt)
+        assert_bits_equal(block, want, "table %d against the oracle" % t)
+    assert not g.takeOobFlag()
+
+
+def test_group_new_buffers_every_call_offsets_out_of_range_ids_and_clones(oracle):
+    """The descriptors are rewritten on every enqueue: new id / offset buffers (and id counts) per
+    call; per-table data_offset with ids outside the shard (skipped and flagged); [1, B] offsets
+    with a trailing end offset; clone and serialize -> deserialize run on the same tables."""
+    rng = np.random.Generator(np.random.PCG64(9))
+    rows, dim, n_bags = [300, 5, 1200], 32, 257
+    shift = [0, 1000, 40]
+    tables = [(rng.standard_normal((r, dim)) * 0.3).astype(np.float32) for r in rows]
+    g = GROUP.createPlugin("sparse", group_fields(tables, 0, [F("offset", np.array(shift, np.int32)),
+                                                             F("include_last_offset", 1), F("xcd_affinity", 0)]))
+    loaded = GROUP.deserializePlugin("sparse", g.serialize())
+    for call, p in enumerate([g, g, g.clone(), loaded]):
+        spill = 3 if call % 2 else 0
+        ids, offs = random_batch(rng, rows, n_bags, np.int32, max_len=5 + 9 * call, lo_spill=spill)
+        ids = [i + s for i, s in zip(ids, shift)]
+        offs = [np.append(o, i.size).astype(np.int32).reshape(1, -1) for o, i in zip(offs, ids)]
+        got = host(p(*[dev(x) for x in interleave(ids, offs)]))
+        any_oob = False
+        for t, tab in enumerate(tables):
+            want, _, n_oob = oracle.embedding_bag(tab, ids[t], offs[t].reshape(-1), 0, include_last_offset=True,
+                                                  data_offset=shift[t])
+            any_oob |= n_oob > 0
+            assert_bits_equal(got[:, t * dim:(t + 1) * dim], want, "call %d table %d" % (call, t))
+        assert p.takeOobFlag() == any_oob
+
+
+def test_group_of_many_tables_and_scaled_config4(oracle):
+    # more tables than one descriptor launch carries (64), odd row width (scalar loads)
+    rng = np.random.Generator(np.random.PCG64(10))
+    rows = [int(r) for r in rng.integers(1, 40, 70)]
+    tables = [rng.standard_normal((r, 6)).astype(np.float32) for r in rows]
+    ids, offs = random_batch(rng, rows, 33, np.int32, max_len=4)
+    got = host(GROUP.createPlugin("many", group_fields(tables, 0))(*[dev(x) for x in interleave(ids, offs)]))
+    for t, tab in enumerate(tables):
+        want, _, _ = oracle.embedding_bag(tab, ids[t], offs[t], 0)
+        assert_bits_equal(got[:, t * 6:(t + 1) * 6], want, "table %d of 70" % t)
+
+    # the 26-table shape at reduced size, fp16 rows and output, with the default cost estimate
+    wl = workloads.config4(variant=3, n_tables=26, n_bags=2048, max_rows=20000)
+    tabs = [wl.host_table(t) for t in range(26)]
+    g = GROUP.createPlugin("sparse", group_fields(tabs, 0, [F("output_fp16", 1)]))
+    got = host(g(*[dev(x) for x in interleave(wl.indices, wl.offsets)]))
+    want = np.zeros((2048, 26 * 128), np.float16)
+    for t in range(26):
+        oracle.embedding_bag(tabs[t], wl.indices[t], wl.offsets[t], oracle.OP_SUM, out=want, out_col=128 * t)
+    assert_bits_equal(got, want, "26 tables through the group plugin")
+
+
+def test_group_enqueue_checks_and_graph_replay(oracle):
+    rng = np.random.Generator(np.random.PCG64(11))
+    rows, dim, n_bags, n_ids = [100, 2000], 16, 64, 500
+    tables = [rng.standard_normal((r, dim)).astype(np.float32) for r in rows]
+    g = GROUP.createPlugin("sparse", group_fields(tables, 0))
+
+    def batch(seed):
+        r = np.random.Generator(np.random.PCG64(seed))
+        ids = [r.integers(0, n, n_ids).astype(np.int32) for n in rows]
+        offs = [np.sort(r.integers(0, n_ids + 1, n_bags)).astype(np.int32) for _ in rows]
+        for o in offs:
+            o[0] = 0
+        return ids, offs
+
+    ids, offs = batch(0)
+    d_in = [dev(x) for x in interleave(ids, offs)]
+    d_out = torch.zeros((n_bags, 2 * dim), dtype=torch.float32, device="cuda")
+    descs = [(tuple(t.shape), lib.I32) for t in d_in]
+    g.configurePlugin(descs, [((n_bags, 2 * dim), lib.F32)])
+    ptrs = [t.data_ptr() for t in d_in]
+    # no workspace, tables that disagree on the bag count: refused before any launch
+    assert g.enqueue_raw(descs, [((n_bags, 2 * dim), lib.F32)], ptrs, [d_out.data_ptr()]) == lib.ERR_BAD_ARG
+    assert "workspace" in lib.last_error()
+    ws = torch.empty(256, dtype=torch.uint8, device="cuda")
+    bad = list(descs)
+    bad[3] = ((n_bags + 1,), lib.I32)
+    rc = g.enqueue_raw(bad, [((n_bags, 2 * dim), lib.F32)], ptrs, [d_out.data_ptr()], workspace_ptr=ws.data_ptr())
+    assert rc == lib.ERR_BAD_ARG and "number of bags" in lib.last_error()
+
+    def want(ids, offs):
+        w = np.zeros((n_bags, 2 * dim), np.float32)
+        for t in range(2):
+            oracle.embedding_bag(tables[t], ids[t], offs[t], 0, out=w, out_col=t * dim)
+        return w
+
+    g.enqueue(d_in, [d_out], workspace=ws)
+    torch.cuda.synchronize()
+    assert_bits_equal(host(d_out), want(ids, offs), "eager")
+    # captured once (descriptor launch + reduction), replayed with new values in the same buffers
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g.enqueue(d_in, [d_out], workspace=ws)
+    for seed in (1, 2, 3):
+        ids, offs = batch(seed)
+        for t, x in zip(d_in, interleave(ids, offs)):
+            t.copy_(torch.from_numpy(x))
+        d_out.fill_(5.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bits_equal(host(d_out), want(ids, offs), "replay %d" % seed)

@@ -19,7 +19,7 @@ def bag_fields(table, op=0, offset=0):
 
 def test_registry_lookup():
     names = {(c.getPluginName(), c.getPluginVersion()) for c in REG.getPluginCreatorList()}
-    assert names == {("EmbeddingBag_TRT", "001"), ("EmbeddingBag_TRT", "002"),
+    assert names == {("EmbeddingBag_TRT", "001"), ("EmbeddingBag_TRT", "002"), ("EmbeddingBagGroup_TRT", "001"),
                      ("ForwardLayerNormPluginDynamic", "1"), ("CustomSkipLayerNormPluginDynamic", "1"),
                      ("CustomEmbLayerNormPluginDynamic", "1")}
     assert REG.getPluginCreator("EmbeddingBag_TRT", "003") is None
@@ -119,6 +119,73 @@ def test_embedding_bag_extended_version():
         c.createPlugin("e", bag_fields(table, op=2) + [F("per_sample_weights", 1)])
     # the five reference fields alone are accepted by the extended creator too
     assert c.createPlugin("e", bag_fields(table.astype(np.float32))).getOutputDataType(0, [lib.I32]) == lib.F32
+
+
+def group_fields(tables, op=0, extra=()):
+    dim = tables[0].shape[1]
+    return [F("dim", dim), F("op", op), F("count", np.array([t.shape[0] for t in tables], np.int32)),
+            F("data", np.concatenate([t.reshape(-1) for t in tables]))] + list(extra)
+
+
+def test_embedding_bag_group_host_contract(tmp_path):
+    rng = np.random.default_rng(5)
+    c = REG.getPluginCreator("EmbeddingBagGroup_TRT", "001")
+    assert [n for n, _ in c.getFieldNames()][:5] == ["dim", "op", "count", "offset", "data"]
+    tables = [rng.standard_normal((r, 8)).astype(np.float16) for r in (3, 7, 2)]
+    p = c.createPlugin("sparse", group_fields(tables, extra=[F("output_fp16", 1), F("index_type", lib.I64),
+                                                             F("offset", np.array([0, 5, 0], np.int32))]))
+    assert p.getPluginType() == "EmbeddingBagGroup_TRT" and p.getPluginVersion() == "001" and p.getNbOutputs() == 1
+    shapes = [(11,), (4,), (0,), (1, 4), (9,), (4,)]
+    assert p.getOutputDimensions(0, shapes) == [4, 24]
+    with pytest.raises(lib.FwdmiError, match="3 tables need 6"):
+        p.getOutputDimensions(0, shapes[:4])
+    with pytest.raises(lib.FwdmiError, match="offsets"):
+        p.getOutputDimensions(0, shapes[:5] + [(5,)])                      # tables disagree on the bag count
+    with pytest.raises(lib.FwdmiError):
+        p.getOutputDimensions(0, [(11, 2)] + shapes[1:])                   # ids must be 1-D
+    io = [(s, lib.I64) for s in shapes] + [((4, 24), lib.F16)]
+    assert all(p.supportsFormatCombination(i, io, 6, 1) for i in range(7))
+    assert not p.supportsFormatCombination(6, io[:6] + [((4, 24), lib.F32)], 6, 1)
+    assert not p.supportsFormatCombination(1, [io[0], ((4,), lib.I32)] + io[2:], 6, 1)
+    assert p.getOutputDataType(0, [lib.I64] * 6) == lib.F16
+    assert p.getWorkspaceSize(io[:6], io[6:]) == 256                       # 3 descriptors of 56 bytes, rounded up
+    blob = p.serialize()
+    head = struct.unpack("<8i", blob[:32])
+    assert head == (8, 0, 3, lib.F16, lib.I64, lib.F16, 0, 1)
+    assert struct.unpack("<3i3i", blob[32:56]) == (3, 7, 2, 0, 5, 0)
+    assert all(x == 1.0 for x in struct.unpack("<3f", blob[56:68]))        # tiny tables: equal cost
+    assert struct.unpack("<Q", blob[68:76]) == (12 * 8,)
+    assert blob[76:] == b"".join(t.tobytes() for t in tables)
+    assert c.deserializePlugin("x", blob).serialize() == blob and p.clone().serialize() == blob
+    for cut in (0, 31, 40, 75, len(blob) - 1):
+        with pytest.raises(lib.FwdmiError):
+            c.deserializePlugin("x", blob[:cut])
+    rc = p.enqueue_raw(io[:6], io[6:], [0] * 6, [0], stream_handle=0)
+    assert rc == lib.ERR_NOT_CONFIGURED
+
+    # contract violations
+    with pytest.raises(lib.FwdmiError, match="required"):
+        c.createPlugin("x", group_fields(tables)[:3])
+    with pytest.raises(lib.FwdmiError, match="dim \\* sum"):
+        c.createPlugin("x", group_fields(tables)[:3] + [F("data", np.zeros(5, np.float16))])
+    with pytest.raises(lib.FwdmiError, match="op must"):
+        c.createPlugin("x", group_fields(tables, op=999))
+    with pytest.raises(lib.FwdmiError, match="one entry per table"):
+        c.createPlugin("x", group_fields(tables, extra=[F("table_cost", np.ones(2, np.float32))]))
+    with pytest.raises(lib.FwdmiError, match="positive"):
+        c.createPlugin("x", group_fields(tables, extra=[F("table_cost", np.array([1, 0, 1], np.float32))]))
+    with pytest.raises(lib.FwdmiError, match="unknown field"):
+        c.createPlugin("x", group_fields(tables, extra=[F("per_sample_weights", 1)]))
+
+    # tables kept by file reference: the blob names the file instead of carrying the rows
+    path = tmp_path / "tables.bin"
+    path.write_bytes(b"".join(t.tobytes() for t in tables))
+    by_ref = c.createPlugin("x", group_fields(tables)[:3] + [
+        F("data_file", np.frombuffer(str(path).encode(), np.int8), lib.FIELD_CHAR),
+        F("table_type", lib.F16)])
+    ref_blob = by_ref.serialize()
+    assert len(ref_blob) == 32 + 36 + 8 + 8 + len(str(path)) + 8 and str(path).encode() in ref_blob
+    assert c.deserializePlugin("x", ref_blob).serialize() == ref_blob
 
 
 def test_enqueue_before_configure_and_wrong_dtype():

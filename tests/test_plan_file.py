@@ -26,7 +26,11 @@ def make_layers(rng):
         F("beta", rng.standard_normal(16).astype(np.float32)), F("gamma", rng.standard_normal(16).astype(np.float32)),
         F("ld", 16), F("type_id", lib.F16)])
     ln.setPluginNamespace("bert")
-    return [("emb_0", bag), ("encoder_layer_0_skip_layer_norm", ln)], t
+    g16 = [rng.standard_normal((r, 8)).astype(np.float16) for r in (4, 9)]
+    group = REG.getPluginCreator("EmbeddingBagGroup_TRT", "001").createPlugin("sparse_stage", [
+        F("dim", 8), F("op", 0), F("count", np.array([4, 9], np.int32)),
+        F("data", np.concatenate([x.reshape(-1) for x in g16])), F("output_fp16", 1)])
+    return [("emb_0", bag), ("encoder_layer_0_skip_layer_norm", ln), ("sparse_stage", group)], t
 
 
 def test_plan_roundtrip_and_sidecar(tmp_path):
@@ -34,7 +38,7 @@ def test_plan_roundtrip_and_sidecar(tmp_path):
     path = str(tmp_path / "engine.plan")
     plugin.save_plan(path, layers, META)
     raw = open(path, "rb").read()
-    assert raw[:8] == b"FWDMIPL1" and struct.unpack("<I", raw[8:12]) == (2,)
+    assert raw[:8] == b"FWDMIPL1" and struct.unpack("<I", raw[8:12]) == (3,)
     assert json.load(open(path + ".meta")) == META           # keys of trt_meta_data.cpp:42-97
     loaded, meta = plugin.load_plan(path)
     assert meta == META and [n for n, _ in loaded] == [n for n, _ in layers]
@@ -113,7 +117,8 @@ def test_plan_load_then_run(tmp_path, oracle):
     assert_bits_equal(host(loaded[0][1](dev(idx), dev(off))), want, "by-value table after load")
     idx2 = rng.integers(0, 500, int(lengths.sum())).astype(np.int32)
     want, _, _ = oracle.embedding_bag(table, idx2, off, 0)
-    assert_bits_equal(host(loaded[2][1](dev(idx2), dev(off))), want, "file-mapped table after load")
+    assert loaded[3][0] == "emb_ref"
+    assert_bits_equal(host(loaded[3][1](dev(idx2), dev(off))), want, "file-mapped table after load")
     x = torch.randn(3, 5, 16, device="cuda", dtype=torch.float16)
     a = layers[1][1](x, x)
     b = loaded[1][1](x, x)

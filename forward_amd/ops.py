@@ -180,6 +180,54 @@ class MultiTableBatch:
         return out
 
 
+def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offset=False, out=None, out_dtype=None,
+                        oob_flag=None, xcd_table_affinity=True, table_cost=None):
+    """All tables of a sparse stage in one launch with this call's ids / offsets:
+    ``[n_bags, T*dim]``, columns ``t*dim ..`` equal to ``embedding_bag(tables[t], indices[t], offsets[t])``.
+
+    The table descriptors go to a device buffer as kernel arguments on torch's current stream
+    (``fwdmi_bag_tables_fill``), so nothing is staged or synchronised on the host.
+    """
+    n = len(tables)
+    _require(n > 0 and len(indices) == n and len(offsets) == n, 'len(tables) == len(indices) == len(offsets) > 0')
+    dim, tdt, idt = tables[0].shape[1], tables[0].dtype, indices[0].dtype
+    n_off = offsets[0].numel()
+    desc = np.zeros((n, 7), np.int64)
+    total = 0
+    for t in range(n):
+        tab, ids, off = _dev(tables[t], "table"), _dev(indices[t], "indices"), _dev(offsets[t], "offsets")
+        _require(tab.dim() == 2 and tab.shape[1] == dim and tab.dtype == tdt, 'tables share dim and dtype')
+        _require(ids.dim() == 1 and ids.dtype == idt and off.dtype == idt, 'ids are 1-D; ids and offsets share a dtype')
+        _require(off.numel() == n_off, 'every table has the same number of offsets')
+        desc[t] = (tab.data_ptr(), ids.data_ptr(), off.data_ptr(), tab.shape[0], ids.numel(), 0, t * dim)
+        total += ids.numel()
+    n_bags = n_off - (1 if include_last_offset else 0)
+    _require(n_bags >= 0, 'offsets hold the trailing end offset when include_last_offset is set')
+    odt = tdt if out_dtype is None else out_dtype
+    if out is None:
+        out = torch.empty((n_bags, n * dim), dtype=odt, device=tables[0].device)
+    _dev(out, "out")
+    _require(out.dtype == odt and out.dim() == 2 and out.shape[0] == n_bags and out.shape[1] >= n * dim,
+             'out is [n_bags, >= T*dim] of the output dtype')
+    cost = None
+    if xcd_table_affinity:
+        if table_cost is None:
+            nbytes = np.array([t.numel() * t.element_size() for t in tables], np.int64)
+            cost = np.empty(n, np.float32)
+            lib.check(lib.dll.fwdmi_bag_table_cost(nbytes.ctypes.data, n, cost.ctypes.data))
+        else:
+            cost = np.ascontiguousarray(table_cost, np.float32)
+            _require(cost.shape == (n,), 'table_cost has one entry per table')
+    d_desc = torch.empty(n * 56, dtype=torch.uint8, device=tables[0].device)
+    s = _stream(None)
+    lib.check(lib.dll.fwdmi_bag_tables_fill(desc.ctypes.data, n, _p(d_desc), s))
+    x = _ext(tables[0], indices[0], odt, include_last_offset=include_last_offset, out_row_stride=out.shape[1],
+             oob_flag=oob_flag, flags=lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0, table_cost=cost)
+    lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(d_desc), n, n_bags, _p(out), dim, _op(mode),
+                                                total / max(1, n_bags * n), C.byref(x), s))
+    return out
+
+
 def _params(gamma, beta, bias=None):
     g, b = _dev(gamma, "gamma"), _dev(beta, "beta")
     _require(g.dtype == torch.float32 and b.dtype == torch.float32,

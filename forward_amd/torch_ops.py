@@ -6,7 +6,7 @@ outputs are copied out of engine buffers; here the ops consume int32 or int64 id
 write straight into the tensors they return.  ``nn.EmbeddingBag`` / ``nn.Embedding`` modules of an
 inference model can be swapped for the HIP path with ``replace_embedding_modules``.
 """
-from typing import Optional
+from typing import List, Optional
 
 import torch
 
@@ -26,6 +26,22 @@ def embedding_bag(weight: torch.Tensor, indices: torch.Tensor, offsets: torch.Te
 def _(weight, indices, offsets, mode, per_sample_weights, include_last_offset):
     n = offsets.numel() - (1 if include_last_offset else 0)
     return weight.new_empty((n, weight.shape[1]))
+
+
+@torch.library.custom_op("fwdmi::embedding_bag_group", mutates_args=())
+def embedding_bag_group(weights: List[torch.Tensor], indices: List[torch.Tensor], offsets: List[torch.Tensor],
+                        mode: int, include_last_offset: bool) -> torch.Tensor:
+    """The embedding bags of a sparse stage and their concatenation: ``[B, T*dim]`` from one launch."""
+    idt = indices[0].dtype
+    return ops.embedding_bag_group(weights, [i.contiguous() for i in indices],
+                                   [o.contiguous().to(idt) for o in offsets], mode,
+                                   include_last_offset=include_last_offset)
+
+
+@embedding_bag_group.register_fake
+def _(weights, indices, offsets, mode, include_last_offset):
+    n = offsets[0].numel() - (1 if include_last_offset else 0)
+    return weights[0].new_empty((n, len(weights) * weights[0].shape[1]))
 
 
 @torch.library.custom_op("fwdmi::embedding_bag_fixed", mutates_args=())
@@ -85,6 +101,34 @@ class EmbeddingBag(torch.nn.Module):
         psw = None if per_sample_weights is None else per_sample_weights.to(self.weight.dtype).contiguous()
         return torch.ops.fwdmi.embedding_bag(self.weight, input, offsets, _MODE[self.mode], psw,
                                              self.include_last_offset)
+
+
+class EmbeddingBagCollection(torch.nn.Module):
+    """The ``nn.EmbeddingBag`` list of a DLRM-style model (equal dim, mode and dtype) as one module:
+    ``forward(indices_list, offsets_list)`` returns what ``torch.cat([bag_t(ids_t, offsets_t)], dim=1)``
+    returns, from one launch."""
+
+    def __init__(self, weights, mode="sum", include_last_offset=False):
+        super().__init__()
+        self.weights = torch.nn.ParameterList(
+            [torch.nn.Parameter(w.detach().contiguous(), requires_grad=False) for w in weights])
+        self.mode, self.include_last_offset = mode, include_last_offset
+
+    @classmethod
+    def from_torch(cls, bags):
+        bags = list(bags)
+        first = bags[0]
+        for m in bags:
+            if m.padding_idx is not None or m.max_norm is not None:
+                raise NotImplementedError("padding_idx / max_norm are not part of the plugin path")
+            if (m.mode, m.include_last_offset, m.embedding_dim, m.weight.dtype) != \
+                    (first.mode, first.include_last_offset, first.embedding_dim, first.weight.dtype):
+                raise ValueError("the bags of a collection share mode, include_last_offset, dim and dtype")
+        return cls([m.weight for m in bags], first.mode, first.include_last_offset)
+
+    def forward(self, indices, offsets):
+        return torch.ops.fwdmi.embedding_bag_group(list(self.weights), list(indices), list(offsets),
+                                                   _MODE[self.mode], self.include_last_offset)
 
 
 class Embedding(torch.nn.Module):

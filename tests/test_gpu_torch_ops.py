@@ -60,3 +60,38 @@ def test_swapped_modules_reproduce_the_reference_dlrm_case(kats):
                              [[-0.18103497, 0.26449448], [-0.25194445, -0.24395032]],
                              [[-0.44896644, -0.45899662], [-0.44896644, -0.45899662]]], axis=1)
     np.testing.assert_allclose(got_bags.cpu().numpy(), expect, atol=1e-4)      # test_torch_dlrm.h:56
+
+
+def test_collection_is_the_concatenation_of_its_bags(kats):
+    # the reference's DLRM case: the three bags as one module, one launch
+    d = kats["dlrm"]
+    model = TinyDlrm([np.array(t, np.float32) for t in d["tables"]]).cuda().eval()
+    idx = [torch.tensor(i, device="cuda") for i in d["indices"]]
+    off = [torch.tensor(o, device="cuda") for o in d["offsets"]]
+    coll = torch_ops.EmbeddingBagCollection.from_torch(model.emb_l)
+    with torch.no_grad():
+        want = torch.cat([m(i, o) for m, i, o in zip(model.emb_l, idx, off)], dim=1)
+        got = coll(idx, off)
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-7)
+    expect = np.concatenate([[[0.48071694, 0.18480009], [0.41585842, -0.29087239]],
+                             [[-0.18103497, 0.26449448], [-0.25194445, -0.24395032]],
+                             [[-0.44896644, -0.45899662], [-0.44896644, -0.45899662]]], axis=1)
+    np.testing.assert_allclose(got.cpu().numpy(), expect, atol=1e-4)           # test_torch_dlrm.h:56
+
+    # a larger stage: every mode and table type, trailing end offsets, against the single-table op bit for bit
+    wl = workloads.config4(variant=6, n_tables=7, n_bags=1500, max_rows=50000)
+    for tdt in (torch.float16, torch.float32):
+        ws = [torch.from_numpy(wl.host_table(t)).cuda().to(tdt) for t in range(7)]
+        ids = [torch.from_numpy(i.astype(np.int64)).cuda() for i in wl.indices]
+        offs = [torch.from_numpy(np.append(o, i.size).astype(np.int64)).cuda() for o, i in zip(wl.offsets, wl.indices)]
+        for mode, code in (("sum", 0), ("mean", 1), ("max", 2)):
+            got = torch.ops.fwdmi.embedding_bag_group(ws, ids, offs, code, True)
+            one = torch.cat([torch.ops.fwdmi.embedding_bag(w, i, o, code, None, True) for w, i, o in zip(ws, ids, offs)], dim=1)
+            assert got.shape == (1500, 7 * 128) and torch.equal(got, one), (tdt, mode)
+            ref = torch.cat([torch.nn.functional.embedding_bag(i, w.float(), o, mode=mode, include_last_offset=True)
+                             for w, i, o in zip(ws, ids, offs)], dim=1)
+            tol = dict(rtol=5e-3, atol=1e-2) if tdt == torch.float16 else dict(rtol=1e-5, atol=1e-6)
+            torch.testing.assert_close(got.float(), ref, **tol)
+    mixed = [torch.nn.EmbeddingBag(5, 4, mode="sum"), torch.nn.EmbeddingBag(5, 4, mode="mean")]
+    with pytest.raises(ValueError):
+        torch_ops.EmbeddingBagCollection.from_torch(mixed)

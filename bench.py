@@ -342,7 +342,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": alg_bytes / launches_per_step,
-                     "kernel_ms_avg": ev_ms / launches_per_step, "kernel_ms_p10": float(np.percentile(per, 10)),
+                     "kernel_ms_avg": ev_ms / launches_per_step, "kernel_ms_median": float(np.median(per)),
+                     "kernel_ms_p10": float(np.percentile(per, 10)),
                      "kernel_ms_p90": float(np.percentile(per, 90)), "launches_per_step": launches_per_step},
         "samples_per_s": wl.n_bags / (ms_per_step * 1e-3),
     }
@@ -350,6 +351,9 @@ def main():
     if os.path.exists(prof) and not args.per_table and args.tables == 26 and args.bags == 65536:
         with open(prof) as f:
             result["roofline"]["traffic"] = json.load(f).get("bag_reduce_config4_bytes_per_launch")
+        if result["roofline"]["traffic"]:
+            # bytes that crossed the L2 boundary (rocprofv3 counters of the same launch) over this run's time
+            result["roofline"]["traffic_GBs"] = result["roofline"]["traffic"] / (ev_ms * 1e-3) / 1e9
 
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()

@@ -7,8 +7,10 @@
 // cross-row shuffles (Chan's parallel Welford update), all in fp32.  gamma / beta (/ bias)
 // live in registers and are reused for every row the wavefront processes.
 //
-// Rows whose length or alignment rule out 128-bit access take the strided kernel: same
-// reduction, one element per lane per step, row read twice (the second time from cache).
+// Rows of at most 512 bytes share a wavefront (64/G rows at a time, G lanes each); rows too long
+// for one wavefront's registers take a workgroup per row.  Rows whose length or alignment rule
+// out 128-bit access take the strided kernel: same reduction, one element per lane per step,
+// row read twice (the second time from cache).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -360,6 +362,152 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
   if (oob && L.oob_flag) atomicOr(L.oob_flag, 1);
 }
 
+// Narrow rows (at most 32 lanes of 16 bytes): a wavefront works on 64/G rows at a time, G lanes
+// per row, so that short rows still fill the 64 lanes.  kLayerNorm / kSkip only.
+template <typename T, int VEC, int MODE>
+__global__ __launch_bounds__(kWG) void ln_narrow_kernel(const LnLaunch L, const int log2_g) {
+  const int lane = threadIdx.x & 63;
+  const int G = 1 << log2_g;
+  const int rows_per_wave = 64 >> log2_g;
+  const int sub = lane >> log2_g;
+  const int gl = lane & (G - 1);
+  const int64_t wave = (int64_t)blockIdx.x * kWavesPerWG + (threadIdx.x >> 6);
+  const T FWDMI_GLOBAL* const in0 = gconst<T>(L.input);
+  const T FWDMI_GLOBAL* const in1 = gconst<T>(L.skip);
+  const bool live = gl * VEC < L.ld;
+  const int col = live ? gl * VEC : 0;
+  const float cnt = live ? (float)VEC : 0.0f;
+  float g[VEC], be[VEC], bi[VEC];
+  {
+    const Pack<float, VEC> pg = gload<float, VEC>(gconst<float>(L.gamma) + col);
+    const Pack<float, VEC> pb = gload<float, VEC>(gconst<float>(L.beta) + col);
+    Pack<float, VEC> pi{};
+    if (L.bias) pi = gload<float, VEC>(gconst<float>(L.bias) + col);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      g[e] = pg.v[e];
+      be[e] = pb.v[e];
+      bi[e] = L.bias ? pi.v[e] : 0.0f;
+    }
+  }
+  const float one = L.one;
+  const int64_t stride = (int64_t)L.total_waves * rows_per_wave;
+  for (int64_t r0 = wave * rows_per_wave; r0 < L.rows; r0 += stride) {
+    const int64_t r = r0 + sub;
+    const bool row_ok = r < L.rows;
+    const int64_t rr = row_ok ? r : L.rows - 1;  // lanes past the last row repeat it and store nothing
+    const Pack<T, VEC> a = gload<T, VEC>(in0 + rr * L.ld + col);
+    Pack<T, VEC> b{};
+    if (MODE == kSkip) b = gload<T, VEC>(in1 + rr * L.ld + col);
+    float x[VEC], sum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      float v = (float)a.v[e];
+      if (MODE == kSkip) v = __builtin_fmaf((float)b.v[e], one, v);
+      x[e] = v + bi[e];
+      sum += live ? x[e] : 0.0f;
+    }
+    Welford w{cnt, sum * (1.0f / (float)VEC), 0.0f};
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float d = live ? x[e] - w.mean : 0.0f;
+      w.m2 = __builtin_fmaf(d, d, w.m2);
+    }
+    for (int m = 1; m < G; m <<= 1) w = merge(w, xor_lanes(w, m));
+    // the lanes of a row agree up to rounding: all take the value of the row's first lane
+    w.n = __shfl(w.n, 0, G);
+    w.mean = __shfl(w.mean, 0, G);
+    w.m2 = __shfl(w.m2, 0, G);
+    const float mu = w.mean;
+    const float rs = __builtin_amdgcn_rsqf(__builtin_fmaf(w.m2, __builtin_amdgcn_rcpf(w.n), L.eps));
+    if (row_ok && live) {
+      Pack<T, VEC> o;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o.v[e] = round_to<T>(__builtin_fmaf(g[e], (x[e] - mu) * rs, be[e]));
+      gstore<T, VEC>(gmut<T>(L.output) + r * L.ld + col, o);
+    }
+  }
+}
+
+// Wide rows (more than 8 slices per lane of a wavefront): a workgroup of 256 lanes owns a row,
+// NV slices per lane in registers (row read once), wavefront statistics merged through LDS.
+// gamma / beta / bias are re-read per row (from cache).  kLayerNorm / kSkip only.
+template <typename T, int VEC, int NV, int MODE>
+__global__ __launch_bounds__(kWG) void ln_block_kernel(const LnLaunch L) {
+  __shared__ float s_part[kWavesPerWG][4];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave_in_wg = tid >> 6;
+  const T FWDMI_GLOBAL* const in0 = gconst<T>(L.input);
+  const T FWDMI_GLOBAL* const in1 = gconst<T>(L.skip);
+  bool live[NV];
+  int col[NV];
+  float cnt = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = (j * kWG + tid) * VEC;
+    live[j] = c < L.ld;
+    col[j] = live[j] ? c : 0;
+    if (live[j]) cnt += (float)VEC;
+  }
+  const float inv_cnt = cnt > 0.0f ? 1.0f / cnt : 0.0f;
+  const float one = L.one;
+  for (int64_t r = blockIdx.x; r < L.rows; r += gridDim.x) {
+    Pack<T, VEC> a[NV], b[MODE == kSkip ? NV : 1];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      a[j] = gload<T, VEC>(in0 + r * L.ld + col[j]);
+      if (MODE == kSkip) b[j] = gload<T, VEC>(in1 + r * L.ld + col[j]);
+    }
+    float x[NV][VEC], sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      Pack<float, VEC> pi{};
+      if (L.bias) pi = gload<float, VEC>(gconst<float>(L.bias) + col[j]);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float v = (float)a[j].v[e];
+        if (MODE == kSkip) v = __builtin_fmaf((float)b[j].v[e], one, v);
+        x[j][e] = v + (L.bias ? pi.v[e] : 0.0f);
+        sum += live[j] ? x[j][e] : 0.0f;
+      }
+    }
+    Welford w{cnt, sum * inv_cnt, 0.0f};
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float d = live[j] ? x[j][e] - w.mean : 0.0f;
+        w.m2 = __builtin_fmaf(d, d, w.m2);
+      }
+    w = wave_allreduce(w);
+    if (lane == 0) {
+      s_part[wave_in_wg][0] = w.n;
+      s_part[wave_in_wg][1] = w.mean;
+      s_part[wave_in_wg][2] = w.m2;
+    }
+    __syncthreads();
+    Welford t{s_part[0][0], s_part[0][1], s_part[0][2]};
+#pragma unroll
+    for (int k = 1; k < kWavesPerWG; ++k) t = merge(t, Welford{s_part[k][0], s_part[k][1], s_part[k][2]});
+    __syncthreads();  // s_part is rewritten for the next row
+    const float mu = t.mean;
+    const float rs = __builtin_amdgcn_rsqf(__builtin_fmaf(t.m2, __builtin_amdgcn_rcpf(t.n), L.eps));
+    T FWDMI_GLOBAL* op = gmut<T>(L.output) + r * L.ld;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      if (live[j]) {
+        const Pack<float, VEC> pg = gload<float, VEC>(gconst<float>(L.gamma) + col[j]);
+        const Pack<float, VEC> pb = gload<float, VEC>(gconst<float>(L.beta) + col[j]);
+        Pack<T, VEC> o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o.v[e] = round_to<T>(__builtin_fmaf(pg.v[e], (x[j][e] - mu) * rs, pb.v[e]));
+        gstore<T, VEC>(op + col[j], o);
+      }
+    }
+  }
+}
+
 // Any ld, any alignment: one element per lane per step, two passes over the row.
 template <typename T, int MODE>
 __global__ __launch_bounds__(kWG) void ln_strided_kernel(const LnLaunch L) {
@@ -440,7 +588,32 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
   const dim3 grid(L.row_blocks + mask_blocks), block(kWG);
 
   const int chunks = (L.ld + 64 * kVec - 1) / (64 * kVec);
-  if (vec_ok && (L.ld % kVec) == 0 && chunks <= 8) {
+  const bool sliceable = vec_ok && (L.ld % kVec) == 0;
+  if constexpr (!is_emb(MODE)) {
+    if (sliceable && L.ld / kVec <= 32) {
+      // several rows per wavefront
+      int log2_g = 0;
+      while ((1 << log2_g) < L.ld / kVec) ++log2_g;
+      const int rows_per_wg = kWavesPerWG * (64 >> log2_g);
+      const int64_t blocks = std::max<int64_t>(1, std::min((L.rows + rows_per_wg - 1) / rows_per_wg, (int64_t)cus * 8));
+      L.total_waves = (int)blocks * kWavesPerWG;
+      hipLaunchKernelGGL((ln_narrow_kernel<T, kVec, MODE>), dim3((unsigned)blocks), block, 0, stream, L, log2_g);
+      FWDMI_HIP_CHECK(hipGetLastError());
+      return FWDMI_OK;
+    }
+    const int block_chunks = (L.ld + kWG * kVec - 1) / (kWG * kVec);
+    if (sliceable && chunks > 8 && block_chunks <= 8) {
+      // a workgroup per row
+      const dim3 bgrid((unsigned)std::max<int64_t>(1, std::min(L.rows, (int64_t)cus * 8)));
+      if (block_chunks <= 4)
+        hipLaunchKernelGGL((ln_block_kernel<T, kVec, 4, MODE>), bgrid, block, 0, stream, L);
+      else
+        hipLaunchKernelGGL((ln_block_kernel<T, kVec, 8, MODE>), bgrid, block, 0, stream, L);
+      FWDMI_HIP_CHECK(hipGetLastError());
+      return FWDMI_OK;
+    }
+  }
+  if (sliceable && chunks <= 8) {
     const int nv = chunks <= 1 ? 1 : chunks <= 2 ? 2 : chunks <= 4 ? 4 : 8;
     const bool full = L.ld == 64 * kVec * nv;
 #define FWDMI_LN_LAUNCH(NV_)                                                                           \

@@ -46,6 +46,7 @@
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #ifdef _OPENMP
@@ -279,18 +280,28 @@ int oracle_skip_layer_norm(int ld, int64_t n, const void* input, const void* ski
                            double eps) {
   if (ld <= 0 || n % ld != 0) return -2;
   int64_t rows = n / ld;
-#pragma omp parallel for schedule(static)
-  for (int64_t r = 0; r < rows; ++r) {
-    double x[16384];
-    for (int i = 0; i < ld; ++i) {
-      double v = load_elem(input, dtype, r * ld + i);
-      if (skip) v += load_elem(skip, dtype, r * ld + i);
-      if (bias) v += bias[i];
-      x[i] = v;
+  int failed = 0;
+#pragma omp parallel
+  {
+    double* x = (double*)malloc(sizeof(double) * (size_t)ld); /* one row, per thread */
+    if (!x) {
+#pragma omp atomic write
+      failed = 1;
     }
-    ln_row(x, ld, gamma, beta, eps, output, dtype, r * (int64_t)ld);
+#pragma omp for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+      if (!x) continue;
+      for (int i = 0; i < ld; ++i) {
+        double v = load_elem(input, dtype, r * ld + i);
+        if (skip) v += load_elem(skip, dtype, r * ld + i);
+        if (bias) v += bias[i];
+        x[i] = v;
+      }
+      ln_row(x, ld, gamma, beta, eps, output, dtype, r * (int64_t)ld);
+    }
+    free(x);
   }
-  return 0;
+  return failed ? -3 : 0;
 }
 
 /*
@@ -307,9 +318,18 @@ int64_t oracle_emb_layer_norm(int S, int B, int ld, const int32_t* input_ids,
                               int tok_count, void* output, int32_t* mask_idx, int dtype,
                               double eps) {
   int64_t oob = 0;
-#pragma omp parallel for schedule(static) reduction(+ : oob)
+  if (ld <= 0) return -2;
+  int failed = 0;
+#pragma omp parallel reduction(+ : oob)
+  {
+  double* x = (double*)malloc(sizeof(double) * (size_t)ld); /* one row, per thread */
+  if (!x) {
+#pragma omp atomic write
+    failed = 1;
+  }
+#pragma omp for schedule(static)
   for (int64_t t = 0; t < (int64_t)S * B; ++t) {
-    double x[16384];
+    if (!x) continue;
     int s = (int)(t / B);
     int64_t w = input_ids[t], g = segment_ids[t];
     int wok = w >= 0 && w < word_count, gok = g >= 0 && g < tok_count, pok = s < pos_count;
@@ -325,6 +345,9 @@ int64_t oracle_emb_layer_norm(int S, int B, int ld, const int32_t* input_ids,
     }
     ln_row(x, ld, gamma, beta, eps, output, dtype, t * (int64_t)ld);
   }
+  free(x);
+  }
+  if (failed) return -3;
   if (mask_idx && input_mask) {
     for (int b = 0; b < B; ++b) {
       int first = S;

@@ -187,4 +187,5 @@ def emb_layer_norm(input_ids, segment_ids, input_mask, word, pos, tok, gamma, be
         _ptr(g), _ptr(word), _ptr(pos), _ptr(tok), ctypes.c_int(word.shape[0]),
         ctypes.c_int(pos.shape[0]), ctypes.c_int(tok.shape[0]), _ptr(out), _ptr(midx),
         ctypes.c_int(_fdt(word)), ctypes.c_double(eps))
+    assert oob >= 0, "oracle_emb_layer_norm failed (%d)" % oob
     return out, midx, int(oob)

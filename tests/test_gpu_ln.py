@@ -60,7 +60,14 @@ def test_config5_emb_then_skip_layer_norm(oracle, dtype):
 @pytest.mark.parametrize("ld,dtype", [(1, np.float32), (7, np.float32), (10, np.float32), (32, np.float16),
                                       (48, np.float32), (100, np.float16), (256, np.float32), (768, np.float32),
                                       (1000, np.float16), (1024, np.float16), (4096, np.float16),
-                                      (2048, np.float32), (5000, np.float32), (8192, np.float16)])
+                                      (2048, np.float32), (5000, np.float32), (8192, np.float16),
+                                      # several rows per wavefront (rows of at most 512 bytes)
+                                      (8, np.float16), (16, np.float16), (64, np.float16), (128, np.float16),
+                                      (248, np.float16), (256, np.float16), (4, np.float32), (128, np.float32),
+                                      # a workgroup per row, and beyond it the strided kernel
+                                      (4104, np.float16), (12000, np.float16), (16384, np.float16),
+                                      (16392, np.float16), (4096, np.float32), (8192, np.float32),
+                                      (8196, np.float32)])
 def test_layer_norm_row_lengths(oracle, ld, dtype):
     rng = np.random.Generator(np.random.PCG64(ld))
     x = (rng.standard_normal((37, ld)) * 2 + 0.5).astype(dtype)
@@ -94,6 +101,15 @@ def test_many_rows_loop_path(oracle):
     g, b = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32), (0.1 * rng.standard_normal(64)).astype(np.float32)
     got = host(ops.layer_norm(dev(x), dev(g), dev(b), eps=1e-5))
     assert_close(got, oracle.layer_norm(x, g, b, eps=1e-5), np.float16)
+
+
+def test_many_wide_rows_loop_path(oracle):
+    rng = np.random.Generator(np.random.PCG64(12))
+    x = rng.standard_normal((2500, 8192)).astype(np.float16)    # more rows than workgroups in the grid
+    sk = rng.standard_normal((2500, 8192)).astype(np.float16)
+    g, b = (1 + 0.1 * rng.standard_normal(8192)).astype(np.float32), (0.1 * rng.standard_normal(8192)).astype(np.float32)
+    got = host(ops.skip_layer_norm(dev(x), dev(g), dev(b), skip=dev(sk), eps=1e-5))
+    assert_close(got, oracle.skip_layer_norm(x, g, b, skip=sk, eps=1e-5), np.float16)
 
 
 def test_emb_layer_norm_mask_and_out_of_table_ids(oracle):

@@ -44,7 +44,8 @@ def parse():
                     help="also run a 1 GiB device-to-device copy (known traffic, to scale rocprof byte counters)")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the benchmark: single-table bag reduction over row widths, table types and "
-                         "bag lengths with uniform random ids, beside torch's GPU embedding_bag (a table on stdout)")
+                         "bag lengths with uniform random ids beside torch's GPU embedding_bag, then SkipLayerNorm "
+                         "over row lengths and counts beside torch's add + layer_norm (two tables on stdout)")
     return ap.parse_args()
 
 
@@ -282,6 +283,29 @@ def sweep(torch, ops):
                         flush=True)
 
 
+def sweep_layer_norm(torch, ops):
+    """SkipLayerNorm (out = LN(x + skip), fp32 gamma / beta) over row lengths, row counts and types;
+    algorithmic bytes = two operands read + one written; beside torch's add + layer_norm on the
+    same GPU, both timed as 10 launches captured in one HIP graph."""
+    print("%7s %6s %5s | %9s %8s | %9s | %s" % ("rows", "ld", "type", "ms", "GB/s", "torch ms", "speedup"), flush=True)
+    for tdt in (torch.float16, torch.float32):
+        for ld in (64, 128, 256, 768, 1000, 1024, 2048, 4096, 8192):
+            for rows in (1024, 8192, 65536, 262144):
+                if rows * ld * 4 > (1 << 30):
+                    continue
+                x = torch.randn((rows, ld), device="cuda").to(tdt)
+                sk = torch.randn((rows, ld), device="cuda").to(tdt)
+                g, b = torch.randn(ld, device="cuda"), torch.randn(ld, device="cuda")
+                out = torch.empty_like(x)
+                ms = time_graph(torch, lambda: ops.skip_layer_norm(x, g, b, skip=sk, eps=1e-5, out=out), inner=10, reps=7)
+                gt, bt = g.to(tdt), b.to(tdt)
+                tms = time_graph(torch, lambda: torch.nn.functional.layer_norm(x + sk, (ld,), gt, bt, 1e-5),
+                                 inner=10, reps=5)
+                nbytes = 3 * rows * ld * x.element_size()
+                print("%7d %6d %5s | %9.4f %8.0f | %9.4f | %.2f" % (
+                    rows, ld, "f16" if tdt == torch.float16 else "f32", ms, nbytes / ms / 1e6, tms, tms / ms), flush=True)
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -295,6 +319,7 @@ def main():
         sys.exit(1)
     if args.sweep:
         sweep(torch, ops)
+        sweep_layer_norm(torch, ops)
         return
 
     t0 = time.time()

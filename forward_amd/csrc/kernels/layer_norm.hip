@@ -601,6 +601,18 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
       FWDMI_HIP_CHECK(hipGetLastError());
       return FWDMI_OK;
     }
+    if (!sliceable && L.ld <= 32) {
+      // rows of at most 32 elements of any alignment (the reference's small-row case,
+      // layer_norm_kernel.cu:285-288): one element per lane, 64/G rows per wavefront
+      int log2_g = 0;
+      while ((1 << log2_g) < L.ld) ++log2_g;
+      const int rows_per_wg = kWavesPerWG * (64 >> log2_g);
+      const int64_t blocks = std::max<int64_t>(1, std::min((L.rows + rows_per_wg - 1) / rows_per_wg, (int64_t)cus * 8));
+      L.total_waves = (int)blocks * kWavesPerWG;
+      hipLaunchKernelGGL((ln_narrow_kernel<T, 1, MODE>), dim3((unsigned)blocks), block, 0, stream, L, log2_g);
+      FWDMI_HIP_CHECK(hipGetLastError());
+      return FWDMI_OK;
+    }
     const int block_chunks = (L.ld + kWG * kVec - 1) / (kWG * kVec);
     if (sliceable && chunks > 8 && block_chunks <= 8) {
       // a workgroup per row

@@ -64,6 +64,7 @@ def test_config5_emb_then_skip_layer_norm(oracle, dtype):
                                       # several rows per wavefront (rows of at most 512 bytes)
                                       (8, np.float16), (16, np.float16), (64, np.float16), (128, np.float16),
                                       (248, np.float16), (256, np.float16), (4, np.float32), (128, np.float32),
+                                      (3, np.float16), (31, np.float16), (25, np.float32), (33, np.float32),
                                       # a workgroup per row, and beyond it the strided kernel
                                       (4104, np.float16), (12000, np.float16), (16384, np.float16),
                                       (16392, np.float16), (4096, np.float32), (8192, np.float32),

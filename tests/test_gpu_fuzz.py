@@ -104,3 +104,29 @@ def test_random_fixed_length_and_gather(oracle, seed):
         got = host(ops.embedding_bag_fixed(dev(table), dev(ids), mode, data_offset=data_offset, oob_flag=flag))
     assert_bits_equal(got.reshape(want.shape), want, "seed %d" % seed)
     assert bool(flag.item()) == (n_oob > 0)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_layer_norm_shapes(oracle, seed):
+    """LayerNorm / SkipLayerNorm over random row lengths (every kernel variant: rows sharing a
+    wavefront, a wavefront per row, a workgroup per row, element-strided), row counts, types and
+    operands, against the float64 oracle at the parity tolerances."""
+    from gpu_util import assert_close
+    r = np.random.Generator(np.random.PCG64(5000 + seed))
+    kind = int(r.integers(0, 5))
+    ld = int([r.integers(1, 33), r.integers(1, 65) * 8, r.integers(33, 2100), r.integers(260, 2050) * 8,
+              r.integers(1, 600) * 2 + 1][kind])
+    rows = int(r.choice([1, 3, 64, 257, 1500]))
+    dt = r.choice([np.float32, np.float16])
+    x = (r.standard_normal((rows, ld)) * r.uniform(0.1, 3.0) + r.uniform(-2, 2)).astype(dt)
+    sk = r.standard_normal((rows, ld)).astype(dt) if r.random() < 0.6 else None
+    bi = (0.1 * r.standard_normal(ld)).astype(np.float32) if r.random() < 0.5 else None
+    g = (1 + 0.1 * r.standard_normal(ld)).astype(np.float32)
+    b = (0.1 * r.standard_normal(ld)).astype(np.float32)
+    eps = float(r.choice([1e-12, 1e-5]))
+    if ld < 4:
+        eps = 1e-5                                  # one or two elements: the variance can be exactly zero
+    got = host(ops.skip_layer_norm(dev(x), dev(g), dev(b), skip=dev(sk), bias=dev(bi), eps=eps))
+    want = oracle.skip_layer_norm(x, g, b, skip=sk, bias=bi, eps=eps)
+    assert got.dtype == dt and got.shape == x.shape
+    assert_close(got, want, dt, scale=4.0)

@@ -61,7 +61,7 @@ enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3, kMaxValue = 4 };
 struct BagLaunch {
   const fwdmi_bag_table* tables;  // device array, or nullptr -> `single`
   fwdmi_bag_table single;
-  const void* psw;  // per-sample weights (single-table form only)
+  const void* psw;  // per-sample weights of the single-table form (a table of a batch carries its own)
   void* out;
   void* max_indices;
   int32_t* oob_flag;
@@ -119,6 +119,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     T.input_size = tp->input_size;
     T.data_offset = tp->data_offset;
     T.out_col = tp->out_col;
+    T.weights = tp->weights;
   } else {
     T = L.single;
   }
@@ -131,7 +132,9 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const int64_t bag0 = (int64_t)wg * L.bags_per_wg;
   const int nb = (int)min((int64_t)L.bags_per_wg, L.n_bags - bag0);
   const TI FWDMI_GLOBAL* __restrict__ ids = gconst<TI>(T.input);
-  const TW FWDMI_GLOBAL* __restrict__ psw = gconst<TW>(L.psw);
+  // per-sample weights: the launch's (single table) or the table's own; none = weight 1
+  const TW FWDMI_GLOBAL* __restrict__ psw = gconst<TW>(L.tables ? T.weights : L.psw);
+  const bool has_w = KIND == kWeighted && (L.tables ? T.weights : L.psw) != nullptr;  // uniform
 
   // ---- stage the run's offsets (clamped) ------------------------------------------------
   for (int i = tid; i <= nb; i += wg_lanes) {
@@ -175,7 +178,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
       } else {
         s_idx[i] = id;
       }
-      if (KIND == kWeighted) s_w[i] = (float)psw[span0 + i];
+      if (KIND == kWeighted) s_w[i] = has_w ? (float)psw[span0 + i] : 1.0f;
     }
   }
   // ---- order the run's bags by length, longest first --------------------------------------
@@ -292,7 +295,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
           w[u] = 0.0f;
           if (!PRED || u < cnt) {
             id[u] = ids[i + u];
-            if (KIND == kWeighted) w[u] = (float)psw[i + u];
+            if (KIND == kWeighted) w[u] = has_w ? (float)psw[i + u] : 1.0f;
           }
         }
       }
@@ -571,12 +574,12 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
 
 // Descriptors of a multi-table batch travel to device memory as kernel arguments: no staging
 // buffer on the host, no copy engine, ordered on the stream like any launch.
-constexpr int kFillChunk = 64;  // 64 x 56 bytes of descriptors per launch, inside the 4 KiB argument limit
+constexpr int kFillChunk = 56;  // 56 x 64 bytes of descriptors per launch, inside the 4 KiB argument limit
 struct TableChunk {
   fwdmi_bag_table t[kFillChunk];
 };
 
-__global__ __launch_bounds__(kFillChunk) void bag_tables_fill_kernel(const TableChunk c, int n,
+__global__ __launch_bounds__(64) void bag_tables_fill_kernel(const TableChunk c, int n,
                                                                      fwdmi_bag_table* dst) {
   const int i = threadIdx.x;
   if (i < n) dst[i] = c.t[i];
@@ -659,7 +662,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   // dim: a row's byte size and a run's (bag, slice) count stay far inside 32 bits
   FWDMI_REQUIRE(n_bags >= 0 && dim > 0 && dim <= (1 << 24) && n_tables > 0,
                 "embedding bag: n_bags=%lld dim=%d (1 .. 2^24) n_tables=%d", (long long)n_bags, dim, n_tables);
-  FWDMI_REQUIRE(!x.per_sample_weights || op == FWDMI_OP_SUM,
+  FWDMI_REQUIRE(!(x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS))) || op == FWDMI_OP_SUM,
                 "embedding bag: per_sample_weights needs op SUM (got %d)", op);
   FWDMI_REQUIRE(!x.max_indices || (op == FWDMI_OP_MAX && !tables_dev),
                 "embedding bag: max_indices needs op MAX on a single table");
@@ -733,7 +736,10 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                 ((out_stride * so) % store_align) == 0 &&
                 (tables_dev || (single.out_col * so) % store_align == 0);
 
-  const int kind = op == FWDMI_OP_MAX ? (x.max_indices ? kMax : kMaxValue) : op == FWDMI_OP_SQUARE_SUM ? kSquare : (x.per_sample_weights ? kWeighted : kPlain);
+  const bool weighted = x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS));
+  const int kind = op == FWDMI_OP_MAX      ? (x.max_indices ? kMax : kMaxValue)
+                   : op == FWDMI_OP_SQUARE_SUM ? kSquare
+                                               : (weighted ? kWeighted : kPlain);
   L.psw = x.per_sample_weights;
   int grid = (int)(wgs * n_tables);
   L.total_wgs = grid;
@@ -788,7 +794,7 @@ extern "C" {
 int fwdmi_embedding_bag(const void* input, const void* input_2, void* output, int64_t input_size,
                         int64_t block_size, const void* data, int64_t count, int32_t dim,
                         int64_t data_offset, int32_t op_type, const fwdmi_bag_ext* ext, void* stream) {
-  fwdmi_bag_table t{data, input, input_2, count, input_size, data_offset, 0};
+  fwdmi_bag_table t{data, input, input_2, count, input_size, data_offset, 0, nullptr};
   const double avg = block_size > 0 ? (double)input_size / (double)block_size : 1.0;
   return fwdmi::bag_dispatch(nullptr, 1, t, output, block_size, -1, dim, op_type, avg, ext,
                              static_cast<hipStream_t>(stream));
@@ -800,7 +806,7 @@ int fwdmi_embedding_bag_fixed(const void* input, void* output, int64_t batch_siz
   if (offset < 0 || batch_size < 0 || (offset > 0 && batch_size > INT64_MAX / offset))
     return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "fixed-length bags: batch %lld x length %lld",
                             (long long)batch_size, (long long)offset);
-  fwdmi_bag_table t{data, input, nullptr, count, batch_size * offset, data_offset, 0};
+  fwdmi_bag_table t{data, input, nullptr, count, batch_size * offset, data_offset, 0, nullptr};
   return fwdmi::bag_dispatch(nullptr, 1, t, output, batch_size, offset, dim, op_type, (double)offset, ext,
                              static_cast<hipStream_t>(stream));
 }
@@ -816,7 +822,7 @@ int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t of
   x.max_indices = nullptr;
   x.out_row_stride = 0;
   const int64_t n = batch_size * offset;
-  fwdmi_bag_table t{data, input, nullptr, count, n, data_offset, 0};
+  fwdmi_bag_table t{data, input, nullptr, count, n, data_offset, 0, nullptr};
   return fwdmi::bag_dispatch(nullptr, 1, t, output, n, 1, dim, FWDMI_OP_SUM, 1.0, &x,
                              static_cast<hipStream_t>(stream));
 }
@@ -826,7 +832,9 @@ int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_table
                               const fwdmi_bag_ext* ext, void* stream) {
   if (!tables_dev) return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "multi-table bags: null table array");
   if (ext && ext->per_sample_weights)
-    return fwdmi::set_error(FWDMI_ERR_UNSUPPORTED, "multi-table bags: per-sample weights are not supported");
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG,
+                            "multi-table bags: per-sample weights go into the table descriptors "
+                            "(FWDMI_BAG_TABLE_WEIGHTS), not into ext->per_sample_weights");
   fwdmi_bag_table none{};
   return fwdmi::bag_dispatch(tables_dev, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, ext,
                              static_cast<hipStream_t>(stream));
@@ -841,7 +849,7 @@ int fwdmi_bag_tables_fill(const fwdmi_bag_table* tables_host, int32_t n_tables, 
     const int n = std::min<int32_t>(fwdmi::kFillChunk, n_tables - at);
     fwdmi::TableChunk c{};
     std::copy(tables_host + at, tables_host + at + n, c.t);
-    hipLaunchKernelGGL(fwdmi::bag_tables_fill_kernel, dim3(1), dim3(fwdmi::kFillChunk), 0,
+    hipLaunchKernelGGL(fwdmi::bag_tables_fill_kernel, dim3(1), dim3(64), 0,
                        static_cast<hipStream_t>(stream), c, n, tables_dev + at);
     FWDMI_HIP_CHECK(hipGetLastError());
   }

@@ -26,6 +26,7 @@ std::string check_spec(const EmbeddingBagGroupSpec& s) {
   if (!is_float_dtype(s.opt.table_dtype) || !is_float_dtype(s.opt.out_dtype) || !is_index_dtype(s.opt.index_dtype))
     return "unsupported table / index / output type";
   if ((int64_t)T * s.dim > INT32_MAX) return "output row too wide";
+  if (s.opt.per_sample_weights && s.op != ReduceOperation::SUM) return "per_sample_weights requires op 0 (sum)";
   return "";
 }
 
@@ -50,22 +51,27 @@ EmbeddingBagGroupPlugin::~EmbeddingBagGroupPlugin() noexcept { terminate(); }
 
 int EmbeddingBagGroupPlugin::getNbOutputs() const noexcept { return 1; }
 
-// 2T inputs (ids_t [N_t], offsets_t [B] or [1, B], the two-input form of
-// embedding_bag_plugin.cpp:84-99 per table) -> [B, T*dim].
+// Per table ids_t [N_t], offsets_t [B] or [1, B] (the two-input form of
+// embedding_bag_plugin.cpp:84-99) and, with per_sample_weights, weights_t [N_t] -> [B, T*dim].
 Dims EmbeddingBagGroupPlugin::getOutputDimensions(int outputIndex, const Dims* inputs, int nbInputs) noexcept {
   clear_error();
   const int T = spec_.n_tables();
-  if (outputIndex != 0 || !inputs || nbInputs != 2 * T) {
+  const int per = inputs_per_table();
+  if (outputIndex != 0 || !inputs || nbInputs != per * T) {
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup: output %d with %d inputs (%d tables need %d)", outputIndex,
-              nbInputs, T, 2 * T);
+              nbInputs, T, per * T);
     return error_dims();
   }
   int64_t n_off = -1;
   for (int t = 0; t < T; ++t) {
-    const Dims& ids = inputs[2 * t];
-    const Dims& off = inputs[2 * t + 1];
+    const Dims& ids = inputs[per * t];
+    const Dims& off = inputs[per * t + 1];
     if (ids.nbDims != 1 || !(off.nbDims == 1 || (off.nbDims == 2 && off.d[0] == 1))) {
       set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup: table %d needs ids [N] and offsets [B] or [1, B]", t);
+      return error_dims();
+    }
+    if (per == 3 && (inputs[per * t + 2].nbDims != 1 || inputs[per * t + 2].d[0] != ids.d[0])) {
+      set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup: table %d needs one weight per id", t);
       return error_dims();
     }
     const int64_t n = off.nbDims == 1 ? off.d[0] : off.d[1];
@@ -85,11 +91,13 @@ Dims EmbeddingBagGroupPlugin::getOutputDimensions(int outputIndex, const Dims* i
 
 bool EmbeddingBagGroupPlugin::supportsFormatCombination(int pos, const PluginTensorDesc* inOut, int nbInputs,
                                                         int nbOutputs) noexcept {
-  if (!inOut || nbInputs != 2 * spec_.n_tables() || nbOutputs != 1 || pos < 0 || pos >= nbInputs + nbOutputs)
+  const int per = inputs_per_table();
+  if (!inOut || nbInputs != per * spec_.n_tables() || nbOutputs != 1 || pos < 0 || pos >= nbInputs + nbOutputs)
     return false;
   const PluginTensorDesc& d = inOut[pos];
   if (d.format != FWDMI_FORMAT_LINEAR) return false;
-  return d.type == (pos >= nbInputs ? spec_.opt.out_dtype : spec_.opt.index_dtype);
+  if (pos >= nbInputs) return d.type == spec_.opt.out_dtype;
+  return d.type == (pos % per == 2 ? spec_.opt.table_dtype : spec_.opt.index_dtype);
 }
 
 // One upload of all tables (one device allocation); clones share it.
@@ -140,6 +148,7 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
   if (!workspace)
     return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup::enqueue needs getWorkspaceSize() bytes of workspace");
   const int T = spec_.n_tables();
+  const int per = inputs_per_table();
   const size_t es = dtype_size(spec_.opt.table_dtype);
   fwdmi_bag_table* const d_tables = static_cast<fwdmi_bag_table*>(workspace);
 
@@ -151,10 +160,10 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
     const int n = std::min(kChunk, T - t0);
     for (int k = 0; k < n; ++k) {
       const int t = t0 + k;
-      if (inputDesc[2 * t].type != spec_.opt.index_dtype || inputDesc[2 * t + 1].type != spec_.opt.index_dtype)
-        return set_error(FWDMI_ERR_UNSUPPORTED, "Unsupported input data type %d", inputDesc[2 * t].type);
-      const Dims& ids = inputDesc[2 * t].dims;
-      const Dims& off = inputDesc[2 * t + 1].dims;
+      if (inputDesc[per * t].type != spec_.opt.index_dtype || inputDesc[per * t + 1].type != spec_.opt.index_dtype)
+        return set_error(FWDMI_ERR_UNSUPPORTED, "Unsupported input data type %d", inputDesc[per * t].type);
+      const Dims& ids = inputDesc[per * t].dims;
+      const Dims& off = inputDesc[per * t + 1].dims;
       if (ids.nbDims != 1 || !(off.nbDims == 1 || (off.nbDims == 2 && off.d[0] == 1)))
         return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup::enqueue: table %d needs ids [N], offsets [B] or [1, B]", t);
       const int64_t no = off.nbDims == 1 ? off.d[0] : off.d[1];
@@ -165,8 +174,17 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
       total_ids += ids.d[0];
       fwdmi_bag_table& d = chunk[k];
       d.data = static_cast<const char*>(d_data_) + row0 * (size_t)spec_.dim * es;
-      d.input = inputs[2 * t];
-      d.input_2 = inputs[2 * t + 1];
+      d.input = inputs[per * t];
+      d.input_2 = inputs[per * t + 1];
+      d.weights = nullptr;
+      if (per == 3) {
+        const PluginTensorDesc& w = inputDesc[per * t + 2];
+        if (w.type != spec_.opt.table_dtype || w.dims.nbDims != 1 || w.dims.d[0] != ids.d[0])
+          return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup::enqueue: table %d needs one weight per id in the table's type", t);
+        d.weights = inputs[per * t + 2];
+        if (ids.d[0] > 0 && !d.weights)
+          return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup::enqueue: null weights (table %d)", t);
+      }
       d.count = spec_.count[t];
       d.input_size = ids.d[0];
       d.data_offset = spec_.offset[t];
@@ -189,7 +207,7 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
   x.include_last_offset = spec_.opt.include_last_offset;
   x.out_row_stride = (int64_t)T * spec_.dim;
   x.oob_flag = d_oob_;
-  x.flags = spec_.xcd_affinity ? FWDMI_BAG_XCD_TABLE_AFFINITY : 0;
+  x.flags = (spec_.xcd_affinity ? FWDMI_BAG_XCD_TABLE_AFFINITY : 0) | (per == 3 ? FWDMI_BAG_TABLE_WEIGHTS : 0);
   x.table_cost = spec_.cost.data();
   const double avg_len = (double)total_ids / ((double)n_bags * T);
   return fwdmi_embedding_bag_multi(d_tables, T, n_bags, outputs[0], spec_.dim, static_cast<int>(spec_.op), avg_len,
@@ -198,11 +216,12 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
 
 // Bytes:
 //   int dim | int op | int T | int table_dtype | int index_dtype | int out_dtype |
-//   int include_last_offset | int xcd_affinity | int count[T] | int offset[T] | float cost[T] |
+//   int include_last_offset | int xcd_affinity | int per_sample_weights |
+//   int count[T] | int offset[T] | float cost[T] |
 //   size_t n | elem[n]                      (all tables back to back), or, for tables given by file,
 //   size_t SIZE_MAX | size_t path_len | path bytes | uint64 byte offset in the file
 size_t EmbeddingBagGroupPlugin::getSerializationSize() const noexcept {
-  const size_t head = 8 * sizeof(int) + (size_t)spec_.n_tables() * (2 * sizeof(int) + sizeof(float)) + sizeof(size_t);
+  const size_t head = 9 * sizeof(int) + (size_t)spec_.n_tables() * (2 * sizeof(int) + sizeof(float)) + sizeof(size_t);
   if (tables_->by_reference()) return head + sizeof(size_t) + tables_->path().size() + sizeof(uint64_t);
   return head + tables_->size();
 }
@@ -217,6 +236,7 @@ void EmbeddingBagGroupPlugin::serialize(void* buffer) const noexcept {
   w.pod<int>(spec_.opt.out_dtype);
   w.pod<int>(spec_.opt.include_last_offset);
   w.pod<int>(spec_.xcd_affinity);
+  w.pod<int>(spec_.opt.per_sample_weights);
   w.bytes(spec_.count.data(), spec_.count.size() * sizeof(int));
   w.bytes(spec_.offset.data(), spec_.offset.size() * sizeof(int));
   w.bytes(spec_.cost.data(), spec_.cost.size() * sizeof(float));
@@ -244,6 +264,7 @@ EmbeddingBagGroupPlugin* EmbeddingBagGroupPlugin::deserialize(const void* data, 
   r.pod(&s.opt.out_dtype);
   r.pod(&s.opt.include_last_offset);
   r.pod(&s.xcd_affinity);
+  r.pod(&s.opt.per_sample_weights);
   if (!r.ok() || T < 1 || T > kMaxGroupTables || r.left() < (size_t)T * (2 * sizeof(int) + sizeof(float))) {
     set_error(FWDMI_ERR_TRUNCATED, "EmbeddingBagGroup: serialized header truncated or malformed");
     return nullptr;
@@ -332,6 +353,7 @@ EmbeddingBagGroupPluginCreator::EmbeddingBagGroupPluginCreator() {
   declare("data_file", PluginFieldType::kCHAR);
   declare("data_file_row_offset", PluginFieldType::kINT32);
   declare("table_type", PluginFieldType::kINT32);
+  declare("per_sample_weights", PluginFieldType::kINT32);
   declare("table_cost", PluginFieldType::kFLOAT32);
   declare("xcd_affinity", PluginFieldType::kINT32);
 }
@@ -361,6 +383,7 @@ IPluginV2DynamicExt* EmbeddingBagGroupPluginCreator::createPlugin(const char*,
     if (name == "dim") scalar = &s.dim, have_dim = true;
     else if (name == "op") scalar = &op, have_op = true;
     else if (name == "include_last_offset") scalar = &s.opt.include_last_offset;
+    else if (name == "per_sample_weights") scalar = &s.opt.per_sample_weights;
     else if (name == "index_type") scalar = &s.opt.index_dtype;
     else if (name == "data_file_row_offset") scalar = &file_row_offset;
     else if (name == "table_type") scalar = &table_type;

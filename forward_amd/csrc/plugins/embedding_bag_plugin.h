@@ -104,7 +104,7 @@ class EmbeddingBagPluginCreatorExt : public EmbeddingBagPluginCreator {
 // launch and write the concatenated [B, T*dim] matrix directly.  It stands for the T
 // EmbeddingBag_TRT layers plus the concatenation layer a DLRM-style graph holds (the reference
 // builds one plugin layer per aten::embedding_bag node, layer_creators/trt_embedding_bag_creator.h:44-85,
-// and concatenates afterwards).  Inputs: ids_0 [N_0], offsets_0 [B] or [1, B], ids_1, offsets_1, ...
+// and concatenates afterwards).  Inputs: ids_0 [N_0], offsets_0 [B] or [1, B] (, weights_0 [N_0]), ids_1, ...
 // Output t*dim .. (t+1)*dim-1 of every row equals what EmbeddingBag_TRT "002" gives for table t.
 constexpr const char* EMBEDDING_BAG_GROUP_PLUGIN_NAME{"EmbeddingBagGroup_TRT"};
 constexpr const char* EMBEDDING_BAG_GROUP_PLUGIN_VERSION{"001"};
@@ -116,7 +116,7 @@ struct EmbeddingBagGroupSpec {
   std::vector<int> count;     // rows per table
   std::vector<int> offset;    // data_offset per table
   std::vector<float> cost;    // relative cost of one bag per table (balances the per-XCD split)
-  EmbeddingBagOptions opt;    // per_sample_weights is not available in a group
+  EmbeddingBagOptions opt;    // per_sample_weights: a third input per table (sum only)
   int xcd_affinity = 1;
   int n_tables() const { return (int)count.size(); }
   size_t total_rows() const {
@@ -158,6 +158,7 @@ class EmbeddingBagGroupPlugin final : public IPluginV2DynamicExt {
   int32_t* oobFlagDevice() const noexcept override { return d_oob_; }
 
  private:
+  int inputs_per_table() const { return spec_.opt.per_sample_weights ? 3 : 2; }
   EmbeddingBagGroupSpec spec_;
   std::shared_ptr<HostDeviceBlob> tables_;  // shared with clones
   void* d_data_ = nullptr;

@@ -24,6 +24,7 @@ FIELD_F16, FIELD_F32, FIELD_F64, FIELD_I8, FIELD_I16, FIELD_I32, FIELD_CHAR, FIE
 FORMAT_LINEAR = 0
 OP_SUM, OP_MEAN, OP_MAX, OP_SQUARE_SUM, OP_GATHER = 0, 1, 2, 3, 999
 BAG_XCD_TABLE_AFFINITY = 1
+BAG_TABLE_WEIGHTS = 2
 
 
 class BagExt(C.Structure):

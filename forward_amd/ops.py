@@ -128,7 +128,7 @@ class MultiTableBatch:
     Holds references to the tables / ids / offsets it points at so they stay alive.
     """
 
-    def __init__(self, tables, indices, offsets, out_cols=None, data_offsets=None):
+    def __init__(self, tables, indices, offsets, out_cols=None, data_offsets=None, per_sample_weights=None):
         _require(len(tables) == len(indices) == len(offsets) and tables,
                  'len(tables) == len(indices) == len(offsets) and tables')
         self.tables = [_dev(t, "table") for t in tables]
@@ -139,15 +139,23 @@ class MultiTableBatch:
         self.n_tables = len(tables)
         out_cols = [t * self.dim for t in range(self.n_tables)] if out_cols is None else list(out_cols)
         data_offsets = [0] * self.n_tables if data_offsets is None else list(data_offsets)
-        desc = np.zeros((self.n_tables, 7), np.int64)
+        psw = [None] * self.n_tables if per_sample_weights is None else list(per_sample_weights)
+        _require(len(psw) == self.n_tables, 'one per_sample_weights entry (or None) per table')
+        self.weights = [None if w is None else _dev(w, "per_sample_weights") for w in psw]
+        self.weighted = any(w is not None for w in self.weights)
+        desc = np.zeros((self.n_tables, 8), np.int64)
         for t in range(self.n_tables):
             _require(self.tables[t].shape[1] == self.dim and self.tables[t].dtype == self.tables[0].dtype,
                      'self.tables[t].shape[1] == self.dim and self.tables[t].dtype == self.tables[0].dtype')
             _require(self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype,
                      'self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype')
             _require(self.offsets[t].numel() == self.n_bags, 'self.offsets[t].numel() == self.n_bags')
+            w = self.weights[t]
+            _require(w is None or (w.dtype == self.tables[t].dtype and w.numel() == self.indices[t].numel()),
+                     'per_sample_weights[t] has the table dtype and one entry per id')
             desc[t] = (self.tables[t].data_ptr(), self.indices[t].data_ptr(), self.offsets[t].data_ptr(),
-                       self.tables[t].shape[0], self.indices[t].numel(), data_offsets[t], out_cols[t])
+                       self.tables[t].shape[0], self.indices[t].numel(), data_offsets[t], out_cols[t],
+                       0 if w is None else w.data_ptr())
         self.width = max(out_cols) + self.dim
         self.total_indices = int(sum(i.numel() for i in self.indices))
         self.desc = torch.from_numpy(desc).to(self.tables[0].device)
@@ -173,7 +181,8 @@ class MultiTableBatch:
             cost = np.ascontiguousarray(cost, np.float32)
             _require(cost.shape == (self.n_tables,), 'cost.shape == (self.n_tables,)')
         x = _ext(self.tables[0], self.indices[0], odt, out_row_stride=out.shape[1], oob_flag=oob_flag,
-                 flags=lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0, table_cost=cost)
+                 flags=(lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0) |
+                       (lib.BAG_TABLE_WEIGHTS if self.weighted else 0), table_cost=cost)
         avg = self.total_indices / max(1, self.n_bags * self.n_tables)
         lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(self.desc), self.n_tables, self.n_bags, _p(out), self.dim,
                                                     _op(mode), avg, C.byref(x), _stream(stream)))
@@ -181,7 +190,7 @@ class MultiTableBatch:
 
 
 def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offset=False, out=None, out_dtype=None,
-                        oob_flag=None, xcd_table_affinity=True, table_cost=None):
+                        oob_flag=None, xcd_table_affinity=True, table_cost=None, per_sample_weights=None):
     """All tables of a sparse stage in one launch with this call's ids / offsets:
     ``[n_bags, T*dim]``, columns ``t*dim ..`` equal to ``embedding_bag(tables[t], indices[t], offsets[t])``.
 
@@ -192,14 +201,22 @@ def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offse
     _require(n > 0 and len(indices) == n and len(offsets) == n, 'len(tables) == len(indices) == len(offsets) > 0')
     dim, tdt, idt = tables[0].shape[1], tables[0].dtype, indices[0].dtype
     n_off = offsets[0].numel()
-    desc = np.zeros((n, 7), np.int64)
+    psw = [None] * n if per_sample_weights is None else list(per_sample_weights)
+    _require(len(psw) == n, 'one per_sample_weights entry (or None) per table')
+    weighted = any(w is not None for w in psw)
+    desc = np.zeros((n, 8), np.int64)
     total = 0
     for t in range(n):
         tab, ids, off = _dev(tables[t], "table"), _dev(indices[t], "indices"), _dev(offsets[t], "offsets")
+        if psw[t] is not None:
+            w = _dev(psw[t], "per_sample_weights")
+            _require(w.dtype == tab.dtype and w.numel() == ids.numel(),
+                     'per_sample_weights[t] has the table dtype and one entry per id')
+            desc[t, 7] = w.data_ptr()
         _require(tab.dim() == 2 and tab.shape[1] == dim and tab.dtype == tdt, 'tables share dim and dtype')
         _require(ids.dim() == 1 and ids.dtype == idt and off.dtype == idt, 'ids are 1-D; ids and offsets share a dtype')
         _require(off.numel() == n_off, 'every table has the same number of offsets')
-        desc[t] = (tab.data_ptr(), ids.data_ptr(), off.data_ptr(), tab.shape[0], ids.numel(), 0, t * dim)
+        desc[t, :7] = (tab.data_ptr(), ids.data_ptr(), off.data_ptr(), tab.shape[0], ids.numel(), 0, t * dim)
         total += ids.numel()
     n_bags = n_off - (1 if include_last_offset else 0)
     _require(n_bags >= 0, 'offsets hold the trailing end offset when include_last_offset is set')
@@ -218,11 +235,12 @@ def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offse
         else:
             cost = np.ascontiguousarray(table_cost, np.float32)
             _require(cost.shape == (n,), 'table_cost has one entry per table')
-    d_desc = torch.empty(n * 56, dtype=torch.uint8, device=tables[0].device)
+    d_desc = torch.empty(n * 64, dtype=torch.uint8, device=tables[0].device)
     s = _stream(None)
     lib.check(lib.dll.fwdmi_bag_tables_fill(desc.ctypes.data, n, _p(d_desc), s))
     x = _ext(tables[0], indices[0], odt, include_last_offset=include_last_offset, out_row_stride=out.shape[1],
-             oob_flag=oob_flag, flags=lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0, table_cost=cost)
+             oob_flag=oob_flag, flags=(lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0) |
+             (lib.BAG_TABLE_WEIGHTS if weighted else 0), table_cost=cost)
     lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(d_desc), n, n_bags, _p(out), dim, _op(mode),
                                                 total / max(1, n_bags * n), C.byref(x), s))
     return out

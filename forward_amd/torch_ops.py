@@ -30,16 +30,21 @@ def _(weight, indices, offsets, mode, per_sample_weights, include_last_offset):
 
 @torch.library.custom_op("fwdmi::embedding_bag_group", mutates_args=())
 def embedding_bag_group(weights: List[torch.Tensor], indices: List[torch.Tensor], offsets: List[torch.Tensor],
-                        mode: int, include_last_offset: bool) -> torch.Tensor:
-    """The embedding bags of a sparse stage and their concatenation: ``[B, T*dim]`` from one launch."""
+                        mode: int, include_last_offset: bool,
+                        per_sample_weights: List[Optional[torch.Tensor]]) -> torch.Tensor:
+    """The embedding bags of a sparse stage and their concatenation: ``[B, T*dim]`` from one launch.
+    ``per_sample_weights``: one entry per table, ``None`` for a table without weights (sum only)."""
     idt = indices[0].dtype
+    psw = [None if w is None else w.to(weights[0].dtype).contiguous() for w in per_sample_weights]
+    if all(w is None for w in psw):
+        psw = None
     return ops.embedding_bag_group(weights, [i.contiguous() for i in indices],
                                    [o.contiguous().to(idt) for o in offsets], mode,
-                                   include_last_offset=include_last_offset)
+                                   include_last_offset=include_last_offset, per_sample_weights=psw)
 
 
 @embedding_bag_group.register_fake
-def _(weights, indices, offsets, mode, include_last_offset):
+def _(weights, indices, offsets, mode, include_last_offset, per_sample_weights):
     n = offsets[0].numel() - (1 if include_last_offset else 0)
     return weights[0].new_empty((n, len(weights) * weights[0].shape[1]))
 
@@ -126,9 +131,10 @@ class EmbeddingBagCollection(torch.nn.Module):
                 raise ValueError("the bags of a collection share mode, include_last_offset, dim and dtype")
         return cls([m.weight for m in bags], first.mode, first.include_last_offset)
 
-    def forward(self, indices, offsets):
+    def forward(self, indices, offsets, per_sample_weights=None):
+        psw = [None] * len(self.weights) if per_sample_weights is None else list(per_sample_weights)
         return torch.ops.fwdmi.embedding_bag_group(list(self.weights), list(indices), list(offsets),
-                                                   _MODE[self.mode], self.include_last_offset)
+                                                   _MODE[self.mode], self.include_last_offset, psw)
 
 
 class Embedding(torch.nn.Module):

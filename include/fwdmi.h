@@ -97,6 +97,10 @@ typedef struct fwdmi_bag_ext {
  * `table_cost` supplies the estimate (large tables whose rows come from HBM cost more per bag
  * than small cache-resident ones), without it all tables count the same. */
 #define FWDMI_BAG_XCD_TABLE_AFFINITY 1
+/* Multi-table launches only (op SUM): every table's descriptor carries a `weights` pointer
+ * (per-sample weights in the table's type, one per id); a table whose pointer is NULL uses
+ * weight 1 for all of its ids. */
+#define FWDMI_BAG_TABLE_WEIGHTS 2
 
 /*
  * Variable-length bags: bag b = input[input_2[b] .. input_2[b+1]), last bag ends at input_size.
@@ -138,6 +142,8 @@ typedef struct fwdmi_bag_table {
   int64_t input_size;
   int64_t data_offset;
   int64_t out_col;     /* first output column of this table's block (a multiple of 8) */
+  const void* weights; /* [input_size] per-sample weights, table dtype; read only with
+                          FWDMI_BAG_TABLE_WEIGHTS; may be NULL */
 } fwdmi_bag_table;
 
 /*
@@ -147,7 +153,8 @@ typedef struct fwdmi_bag_table {
  * with ext->out_row_stride set (the reference issues one plugin enqueue per table,
  * embedding_bag_plugin.cpp:146-189, and concatenates afterwards).
  * `avg_bag_len` (>0) is a sizing hint: the mean ids per bag over the batch.
- * Per-sample weights and max_indices are not available in this form.
+ * Per-sample weights come through the descriptors (FWDMI_BAG_TABLE_WEIGHTS), not through
+ * ext->per_sample_weights; max_indices is not available in this form.
  */
 int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_tables, int64_t n_bags,
                               void* output, int32_t dim, int32_t op_type, double avg_bag_len,

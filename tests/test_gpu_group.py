@@ -83,7 +83,7 @@ def test_group_new_buffers_every_call_offsets_out_of_range_ids_and_clones(oracle
 
 
 def test_group_of_many_tables_and_scaled_config4(oracle):
-    # more tables than one descriptor launch carries (64), odd row width (scalar loads)
+    # more tables than one descriptor launch carries (56), odd row width (scalar loads)
     rng = np.random.Generator(np.random.PCG64(10))
     rows = [int(r) for r in rng.integers(1, 40, 70)]
     tables = [rng.standard_normal((r, 6)).astype(np.float32) for r in rows]
@@ -154,3 +154,29 @@ def test_group_enqueue_checks_and_graph_replay(oracle):
         graph.replay()
         torch.cuda.synchronize()
         assert_bits_equal(host(d_out), want(ids, offs), "replay %d" % seed)
+
+
+@pytest.mark.parametrize("tdt", [np.float16, np.float32])
+def test_group_with_per_sample_weights(oracle, tdt):
+    rng = np.random.Generator(np.random.PCG64(12))
+    rows, dim, n_bags = [40, 3000, 700], 64, 500
+    tables = [(rng.standard_normal((r, dim)) * 0.3).astype(tdt) for r in rows]
+    ids, offs = random_batch(rng, rows, n_bags, np.int32, max_len=30)
+    psw = [rng.random(i.size).astype(tdt) for i in ids]
+    g = GROUP.createPlugin("sparse", group_fields(tables, 0, [F("per_sample_weights", 1)]))
+    ins = [x for trio in zip(ids, offs, psw) for x in trio]
+    got = host(g(*[dev(x) for x in ins]))
+    for t, tab in enumerate(tables):
+        want, _, _ = oracle.embedding_bag(tab, ids[t], offs[t], 0, per_sample_weights=psw[t], out_dtype=np.float32)
+        assert_bits_equal(got[:, t * dim:(t + 1) * dim], want, "weighted table %d" % t)
+    # the launcher form: weights on some tables only (the others count every id once)
+    from forward_amd import ops
+    batch = ops.MultiTableBatch([dev(t) for t in tables], [dev(i) for i in ids], [dev(o) for o in offs],
+                                per_sample_weights=[dev(psw[0]), None, dev(psw[2])])
+    out = host(batch.forward(out_dtype=torch.float32, xcd_table_affinity=True))
+    for t, tab in enumerate(tables):
+        want, _, _ = oracle.embedding_bag(tab, ids[t], offs[t], 0, per_sample_weights=None if t == 1 else psw[t],
+                                          out_dtype=np.float32)
+        assert_bits_equal(out[:, t * dim:(t + 1) * dim], want, "launcher, table %d" % t)
+    with pytest.raises(lib.FwdmiError, match="SUM"):
+        batch.forward(mode="max")

@@ -85,13 +85,18 @@ def test_collection_is_the_concatenation_of_its_bags(kats):
         ids = [torch.from_numpy(i.astype(np.int64)).cuda() for i in wl.indices]
         offs = [torch.from_numpy(np.append(o, i.size).astype(np.int64)).cuda() for o, i in zip(wl.offsets, wl.indices)]
         for mode, code in (("sum", 0), ("mean", 1), ("max", 2)):
-            got = torch.ops.fwdmi.embedding_bag_group(ws, ids, offs, code, True)
+            got = torch.ops.fwdmi.embedding_bag_group(ws, ids, offs, code, True, [None] * 7)
             one = torch.cat([torch.ops.fwdmi.embedding_bag(w, i, o, code, None, True) for w, i, o in zip(ws, ids, offs)], dim=1)
             assert got.shape == (1500, 7 * 128) and torch.equal(got, one), (tdt, mode)
             ref = torch.cat([torch.nn.functional.embedding_bag(i, w.float(), o, mode=mode, include_last_offset=True)
                              for w, i, o in zip(ws, ids, offs)], dim=1)
             tol = dict(rtol=5e-3, atol=1e-2) if tdt == torch.float16 else dict(rtol=1e-5, atol=1e-6)
             torch.testing.assert_close(got.float(), ref, **tol)
+        # per-sample weights on some of the tables only
+        psw = [torch.rand(i.numel(), device="cuda").to(tdt) if t % 2 == 0 else None for t, i in enumerate(ids)]
+        got = torch.ops.fwdmi.embedding_bag_group(ws, ids, offs, 0, True, psw)
+        one = torch.cat([torch.ops.fwdmi.embedding_bag(w, i, o, 0, p, True) for w, i, o, p in zip(ws, ids, offs, psw)], dim=1)
+        assert torch.equal(got, one), (tdt, "weighted")
     mixed = [torch.nn.EmbeddingBag(5, 4, mode="sum"), torch.nn.EmbeddingBag(5, 4, mode="mean")]
     with pytest.raises(ValueError):
         torch_ops.EmbeddingBagCollection.from_torch(mixed)

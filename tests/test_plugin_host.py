@@ -148,16 +148,16 @@ def test_embedding_bag_group_host_contract(tmp_path):
     assert not p.supportsFormatCombination(6, io[:6] + [((4, 24), lib.F32)], 6, 1)
     assert not p.supportsFormatCombination(1, [io[0], ((4,), lib.I32)] + io[2:], 6, 1)
     assert p.getOutputDataType(0, [lib.I64] * 6) == lib.F16
-    assert p.getWorkspaceSize(io[:6], io[6:]) == 256                       # 3 descriptors of 56 bytes, rounded up
+    assert p.getWorkspaceSize(io[:6], io[6:]) == 256                       # 3 descriptors of 64 bytes, rounded up
     blob = p.serialize()
-    head = struct.unpack("<8i", blob[:32])
-    assert head == (8, 0, 3, lib.F16, lib.I64, lib.F16, 0, 1)
-    assert struct.unpack("<3i3i", blob[32:56]) == (3, 7, 2, 0, 5, 0)
-    assert all(x == 1.0 for x in struct.unpack("<3f", blob[56:68]))        # tiny tables: equal cost
-    assert struct.unpack("<Q", blob[68:76]) == (12 * 8,)
-    assert blob[76:] == b"".join(t.tobytes() for t in tables)
+    head = struct.unpack("<9i", blob[:36])
+    assert head == (8, 0, 3, lib.F16, lib.I64, lib.F16, 0, 1, 0)
+    assert struct.unpack("<3i3i", blob[36:60]) == (3, 7, 2, 0, 5, 0)
+    assert all(x == 1.0 for x in struct.unpack("<3f", blob[60:72]))        # tiny tables: equal cost
+    assert struct.unpack("<Q", blob[72:80]) == (12 * 8,)
+    assert blob[80:] == b"".join(t.tobytes() for t in tables)
     assert c.deserializePlugin("x", blob).serialize() == blob and p.clone().serialize() == blob
-    for cut in (0, 31, 40, 75, len(blob) - 1):
+    for cut in (0, 35, 44, 79, len(blob) - 1):
         with pytest.raises(lib.FwdmiError):
             c.deserializePlugin("x", blob[:cut])
     rc = p.enqueue_raw(io[:6], io[6:], [0] * 6, [0], stream_handle=0)
@@ -175,7 +175,19 @@ def test_embedding_bag_group_host_contract(tmp_path):
     with pytest.raises(lib.FwdmiError, match="positive"):
         c.createPlugin("x", group_fields(tables, extra=[F("table_cost", np.array([1, 0, 1], np.float32))]))
     with pytest.raises(lib.FwdmiError, match="unknown field"):
-        c.createPlugin("x", group_fields(tables, extra=[F("per_sample_weights", 1)]))
+        c.createPlugin("x", group_fields(tables, extra=[F("max_norm", 1)]))
+    with pytest.raises(lib.FwdmiError, match="requires op 0"):
+        c.createPlugin("x", group_fields(tables, op=2, extra=[F("per_sample_weights", 1)]))
+    # per-sample weights: a third input per table, in the table's type
+    w = c.createPlugin("x", group_fields(tables, extra=[F("per_sample_weights", 1)]))
+    wshapes = [(11,), (4,), (11,), (0,), (4,), (0,), (9,), (4,), (9,)]
+    assert w.getOutputDimensions(0, wshapes) == [4, 24]
+    with pytest.raises(lib.FwdmiError, match="one weight per id"):
+        w.getOutputDimensions(0, wshapes[:2] + [(10,)] + wshapes[3:])
+    wio = [(s_, lib.F16 if i % 3 == 2 else lib.I32) for i, s_ in enumerate(wshapes)] + [((4, 24), lib.F32)]
+    assert all(w.supportsFormatCombination(i, wio, 9, 1) for i in range(10))
+    assert not w.supportsFormatCombination(2, wio[:2] + [((11,), lib.F32)] + wio[3:], 9, 1)
+    assert struct.unpack("<9i", w.serialize()[:36])[8] == 1
 
     # tables kept by file reference: the blob names the file instead of carrying the rows
     path = tmp_path / "tables.bin"
@@ -184,7 +196,7 @@ def test_embedding_bag_group_host_contract(tmp_path):
         F("data_file", np.frombuffer(str(path).encode(), np.int8), lib.FIELD_CHAR),
         F("table_type", lib.F16)])
     ref_blob = by_ref.serialize()
-    assert len(ref_blob) == 32 + 36 + 8 + 8 + len(str(path)) + 8 and str(path).encode() in ref_blob
+    assert len(ref_blob) == 36 + 36 + 8 + 8 + len(str(path)) + 8 and str(path).encode() in ref_blob
     assert c.deserializePlugin("x", ref_blob).serialize() == ref_blob
 
 

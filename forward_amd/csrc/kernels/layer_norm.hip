@@ -8,9 +8,10 @@
 // live in registers and are reused for every row the wavefront processes.
 //
 // Rows of at most 512 bytes share a wavefront (64/G rows at a time, G lanes each); rows too long
-// for one wavefront's registers take a workgroup per row.  Rows whose length or alignment rule
-// out 128-bit access take the strided kernel: same reduction, one element per lane per step,
-// row read twice (the second time from cache).
+// for one wavefront's registers take a workgroup per row, and so do rows whose length or
+// alignment rule out 128-bit access (one element per lane per slice).  What is left (rows beyond
+// a workgroup's registers, embedding rows without 128-bit access) takes the strided kernel: same
+// reduction, one element per lane per step, row read twice (the second time from cache).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -621,6 +622,35 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
         hipLaunchKernelGGL((ln_block_kernel<T, kVec, 4, MODE>), bgrid, block, 0, stream, L);
       else
         hipLaunchKernelGGL((ln_block_kernel<T, kVec, 8, MODE>), bgrid, block, 0, stream, L);
+      FWDMI_HIP_CHECK(hipGetLastError());
+      return FWDMI_OK;
+    }
+    // Rows that cannot be cut into 16-byte slices (odd length or unaligned operands) are still read
+    // once, one element per lane per slice: a wavefront per row up to 512 elements, a workgroup
+    // per row up to 8192.
+    if (!sliceable && L.ld <= 64 * 8) {
+      const int nv1 = L.ld <= 64 ? 1 : L.ld <= 128 ? 2 : L.ld <= 256 ? 4 : 8;
+      if (nv1 == 1)
+        hipLaunchKernelGGL((ln_rows_kernel<T, 1, 1, MODE, false>), grid, block, 0, stream, L);
+      else if (nv1 == 2)
+        hipLaunchKernelGGL((ln_rows_kernel<T, 1, 2, MODE, false>), grid, block, 0, stream, L);
+      else if (nv1 == 4)
+        hipLaunchKernelGGL((ln_rows_kernel<T, 1, 4, MODE, false>), grid, block, 0, stream, L);
+      else
+        hipLaunchKernelGGL((ln_rows_kernel<T, 1, 8, MODE, false>), grid, block, 0, stream, L);
+      FWDMI_HIP_CHECK(hipGetLastError());
+      return FWDMI_OK;
+    }
+    if (!sliceable && L.ld <= kWG * 32) {
+      const dim3 bgrid((unsigned)std::max<int64_t>(1, std::min(L.rows, (int64_t)cus * 8)));
+      if (L.ld <= kWG * 4)
+        hipLaunchKernelGGL((ln_block_kernel<T, 1, 4, MODE>), bgrid, block, 0, stream, L);
+      else if (L.ld <= kWG * 8)
+        hipLaunchKernelGGL((ln_block_kernel<T, 1, 8, MODE>), bgrid, block, 0, stream, L);
+      else if (L.ld <= kWG * 16)
+        hipLaunchKernelGGL((ln_block_kernel<T, 1, 16, MODE>), bgrid, block, 0, stream, L);
+      else
+        hipLaunchKernelGGL((ln_block_kernel<T, 1, 32, MODE>), bgrid, block, 0, stream, L);
       FWDMI_HIP_CHECK(hipGetLastError());
       return FWDMI_OK;
     }

@@ -65,6 +65,9 @@ def test_config5_emb_then_skip_layer_norm(oracle, dtype):
                                       (8, np.float16), (16, np.float16), (64, np.float16), (128, np.float16),
                                       (248, np.float16), (256, np.float16), (4, np.float32), (128, np.float32),
                                       (3, np.float16), (31, np.float16), (25, np.float32), (33, np.float32),
+                                      # no 16-byte slices: one element per lane, a workgroup per row
+                                      (513, np.float32), (1001, np.float16), (2050, np.float16), (8191, np.float32),
+                                      (8193, np.float32),
                                       # a workgroup per row, and beyond it the strided kernel
                                       (4104, np.float16), (12000, np.float16), (16384, np.float16),
                                       (16392, np.float16), (4096, np.float32), (8192, np.float32),
@@ -102,6 +105,20 @@ def test_many_rows_loop_path(oracle):
     g, b = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32), (0.1 * rng.standard_normal(64)).astype(np.float32)
     got = host(ops.layer_norm(dev(x), dev(g), dev(b), eps=1e-5))
     assert_close(got, oracle.layer_norm(x, g, b, eps=1e-5), np.float16)
+
+
+def test_unaligned_operands(oracle):
+    """Operands that start one element into a buffer: no 128-bit access, same results."""
+    rng = np.random.Generator(np.random.PCG64(13))
+    for dtype, ld in ((np.float16, 1024), (np.float32, 768), (np.float16, 16)):
+        x = rng.standard_normal((50, ld)).astype(dtype)
+        sk = rng.standard_normal((50, ld)).astype(dtype)
+        g, b = (1 + 0.1 * rng.standard_normal(ld)).astype(np.float32), (0.1 * rng.standard_normal(ld)).astype(np.float32)
+        shifted = lambda a: dev(np.concatenate([[0], a.reshape(-1)]).astype(a.dtype))[1:].reshape(a.shape)
+        dx, dsk = shifted(x), shifted(sk)
+        assert dx.data_ptr() % 16 != 0 and dx.is_contiguous()
+        got = host(ops.skip_layer_norm(dx, dev(g), dev(b), skip=dsk, eps=1e-5))
+        assert_close(got, oracle.skip_layer_norm(x, g, b, skip=sk, eps=1e-5), dtype)
 
 
 def test_many_wide_rows_loop_path(oracle):

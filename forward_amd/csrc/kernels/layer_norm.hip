@@ -364,20 +364,27 @@ __global__ __launch_bounds__(kWG) void ln_rows_kernel(const LnLaunch L) {
 }
 
 // Narrow rows (at most 32 lanes of 16 bytes): a wavefront works on 64/G rows at a time, G lanes
-// per row, so that short rows still fill the 64 lanes.  kLayerNorm / kSkip only.
+// per row, so that short rows still fill the 64 lanes.  kLayerNorm / kSkip / kEmb.
 template <typename T, int VEC, int MODE>
 __global__ __launch_bounds__(kWG) void ln_narrow_kernel(const LnLaunch L, const int log2_g) {
   const int lane = threadIdx.x & 63;
+  if (MODE == kEmb && (int)blockIdx.x >= L.row_blocks) {
+    const int b = ((int)blockIdx.x - L.row_blocks) * kWavesPerWG + (threadIdx.x >> 6);
+    if (b < L.B) mask_index_wave(L, b, lane);
+    return;
+  }
   const int G = 1 << log2_g;
   const int rows_per_wave = 64 >> log2_g;
   const int sub = lane >> log2_g;
   const int gl = lane & (G - 1);
   const int64_t wave = (int64_t)blockIdx.x * kWavesPerWG + (threadIdx.x >> 6);
   const T FWDMI_GLOBAL* const in0 = gconst<T>(L.input);
-  const T FWDMI_GLOBAL* const in1 = gconst<T>(L.skip);
+  const T FWDMI_GLOBAL* const in1 = gconst<T>(MODE == kEmb ? L.pos : L.skip);
+  const T FWDMI_GLOBAL* const in2 = gconst<T>(L.tok);
   const bool live = gl * VEC < L.ld;
   const int col = live ? gl * VEC : 0;
   const float cnt = live ? (float)VEC : 0.0f;
+  bool oob = false;
   float g[VEC], be[VEC], bi[VEC];
   {
     const Pack<float, VEC> pg = gload<float, VEC>(gconst<float>(L.gamma) + col);
@@ -397,15 +404,27 @@ __global__ __launch_bounds__(kWG) void ln_narrow_kernel(const LnLaunch L, const 
     const int64_t r = r0 + sub;
     const bool row_ok = r < L.rows;
     const int64_t rr = row_ok ? r : L.rows - 1;  // lanes past the last row repeat it and store nothing
-    const Pack<T, VEC> a = gload<T, VEC>(in0 + rr * L.ld + col);
-    Pack<T, VEC> b{};
-    if (MODE == kSkip) b = gload<T, VEC>(in1 + rr * L.ld + col);
+    Pack<T, VEC> a{}, b{}, c{};
+    if (MODE == kEmb) {
+      // word + position + token-type rows of token rr; an id outside its table contributes zeros
+      const int s = L.batch_major ? (int)(rr % L.S) : (int)(rr / L.B);
+      const int64_t w = L.input_ids[rr], sg = L.segment_ids[rr];
+      const bool ok0 = w >= 0 && w < L.word_count, ok1 = s < L.pos_count, ok2 = sg >= 0 && sg < L.tok_count;
+      oob |= row_ok && !(ok0 && ok1 && ok2);
+      if (ok0) a = gload<T, VEC>(in0 + w * L.ld + col);
+      if (ok1) b = gload<T, VEC>(in1 + (int64_t)s * L.ld + col);
+      if (ok2) c = gload<T, VEC>(in2 + sg * L.ld + col);
+    } else {
+      a = gload<T, VEC>(in0 + rr * L.ld + col);
+      if (MODE == kSkip) b = gload<T, VEC>(in1 + rr * L.ld + col);
+    }
     float x[VEC], sum = 0.0f;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
       float v = (float)a.v[e];
-      if (MODE == kSkip) v = __builtin_fmaf((float)b.v[e], one, v);
-      x[e] = v + bi[e];
+      if (MODE != kLayerNorm) v = __builtin_fmaf((float)b.v[e], one, v);
+      if (MODE == kEmb) v = __builtin_fmaf((float)c.v[e], one, v);
+      x[e] = MODE == kEmb ? v : v + bi[e];
       sum += live ? x[e] : 0.0f;
     }
     Welford w{cnt, sum * (1.0f / (float)VEC), 0.0f};
@@ -428,6 +447,7 @@ __global__ __launch_bounds__(kWG) void ln_narrow_kernel(const LnLaunch L, const 
       gstore<T, VEC>(gmut<T>(L.output) + r * L.ld + col, o);
     }
   }
+  if (MODE == kEmb && oob && L.oob_flag) atomicOr(L.oob_flag, 1);
 }
 
 // Wide rows (more than 8 slices per lane of a wavefront): a workgroup of 256 lanes owns a row,
@@ -590,6 +610,21 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
 
   const int chunks = (L.ld + 64 * kVec - 1) / (64 * kVec);
   const bool sliceable = vec_ok && (L.ld % kVec) == 0;
+  if constexpr (MODE == kEmb) {
+    if (sliceable && L.ld / kVec <= 32) {
+      // several tokens per wavefront (hidden sizes of at most 512 bytes)
+      int log2_g = 0;
+      while ((1 << log2_g) < L.ld / kVec) ++log2_g;
+      const int rows_per_wg = kWavesPerWG * (64 >> log2_g);
+      const int64_t blocks = std::max<int64_t>(1, std::min((L.rows + rows_per_wg - 1) / rows_per_wg, (int64_t)cus * 8));
+      L.row_blocks = (int)blocks;
+      L.total_waves = (int)blocks * kWavesPerWG;
+      hipLaunchKernelGGL((ln_narrow_kernel<T, kVec, MODE>), dim3((unsigned)(blocks + mask_blocks)), block, 0, stream, L,
+                         log2_g);
+      FWDMI_HIP_CHECK(hipGetLastError());
+      return FWDMI_OK;
+    }
+  }
   if constexpr (!is_emb(MODE)) {
     if (sliceable && L.ld / kVec <= 32) {
       // several rows per wavefront
@@ -682,10 +717,13 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
   return FWDMI_OK;
 }
 
-// True when rows of `ld` elements of `dtype` can take the register-resident kernel.
+// True when rows of `ld` elements of `dtype` take the wavefront-per-row kernel in every mode, so
+// that the fused embedding + skip form rounds exactly like its two separate launches.  (Rows of
+// at most 512 bytes take the several-rows-per-wavefront kernel when launched separately; their
+// fused form is issued as those two launches.)
 bool rows_kernel_ok(int ld, int dtype, bool vec_ok) {
   const int vec = 16 / (int)dtype_size(dtype);
-  return vec_ok && ld % vec == 0 && (ld + 64 * vec - 1) / (64 * vec) <= 8;
+  return vec_ok && ld % vec == 0 && ld / vec > 32 && (ld + 64 * vec - 1) / (64 * vec) <= 8;
 }
 
 template <int MODE>
@@ -772,8 +810,8 @@ int fwdmi_emb_layer_norm_ex(void* stream, int32_t S, int32_t B, int32_t ld, cons
   L.eps = eps;
   L.batch_major = ext && ext->batch_major;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  bool vec_ok = aligned16(word) && aligned16(pos) && aligned16(tok) && aligned16(output) && aligned16(gamma) &&
-                aligned16(beta);
+  const bool tables_ok = aligned16(word) && aligned16(pos) && aligned16(tok) && aligned16(gamma) && aligned16(beta);
+  bool vec_ok = tables_ok && aligned16(output);
   if (!fused) return ln_dispatch<kEmb>(L, dtype, vec_ok, s);
 
   vec_ok = vec_ok && aligned16(ext->skip) && aligned16(ext->gamma2) && aligned16(ext->beta2) &&
@@ -787,10 +825,10 @@ int fwdmi_emb_layer_norm_ex(void* stream, int32_t S, int32_t B, int32_t ld, cons
     L.emb_output = ext->emb_output;
     return ln_dispatch<kEmbSkip>(L, dtype, vec_ok, s);
   }
-  // rows that cannot stay in registers: two launches, the second in place over the first result
+  // every other row shape: the two launches themselves, the second in place over the first result
   void* first = ext->emb_output ? ext->emb_output : output;
   L.output = first;
-  int rc = ln_dispatch<kEmb>(L, dtype, false, s);
+  int rc = ln_dispatch<kEmb>(L, dtype, tables_ok && aligned16(first), s);
   if (rc != FWDMI_OK) return rc;
   return fwdmi_skip_layer_norm(stream, ld, (int64_t)S * B * ld, first, ext->skip, ext->beta2, ext->gamma2, output,
                                ext->bias2, dtype, ext->eps2);

@@ -269,7 +269,42 @@ def test_batch_major_layout_equals_transposed_sequence_major(oracle, dtype):
     np.testing.assert_array_equal(host(e2), host(e))
 
 
-@pytest.mark.parametrize("dtype,hidden", [(np.float16, 1024), (np.float32, 1024), (np.float16, 768), (np.float16, 100)])
+@pytest.mark.parametrize("dtype,hidden", [(np.float16, 128), (np.float16, 256), (np.float32, 64), (np.float32, 128),
+                                          (np.float16, 8)])
+def test_small_hidden_sizes_share_a_wavefront(oracle, dtype, hidden):
+    """BERT-tiny / -mini sized embeddings: several tokens per wavefront.  Values against the oracle,
+    mask index and out-of-table ids exactly, batch-major equal to the transposed sequence-major run."""
+    rng = np.random.Generator(np.random.PCG64(100 + hidden))
+    S, B, V, P = 37, 9, 500, 40
+    mk = lambda *s, mu=0.0, sd=0.02: (mu + sd * rng.standard_normal(s)).astype(np.float32).astype(dtype)
+    word, pos, tok = mk(V, hidden), mk(P, hidden), mk(2, hidden)
+    g, b = mk(hidden, mu=1.0).astype(np.float32), mk(hidden).astype(np.float32)
+    ids = rng.integers(0, V, (S, B)).astype(np.int32)
+    seg = rng.integers(0, 2, (S, B)).astype(np.int32)
+    lens = rng.integers(1, S + 1, B)
+    msk = (np.arange(S)[:, None] < lens[None, :]).astype(np.int32)
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    tabs = [dev(word), dev(pos), dev(tok), dev(g), dev(b)]
+    got, midx = ops.emb_layer_norm(dev(ids), dev(seg), dev(msk), *tabs, eps=1e-12, oob_flag=flag)
+    want, wmidx, n_oob = oracle.emb_layer_norm(ids, seg, msk, word, pos, tok, g, b, eps=1e-12)
+    assert n_oob == 0 and not flag.item()
+    assert_close(host(got), want, dtype)
+    np.testing.assert_array_equal(host(midx), wmidx)
+    t = lambda x: np.ascontiguousarray(x.T)
+    bm, bmidx = ops.emb_layer_norm(dev(t(ids)), dev(t(seg)), dev(t(msk)), *tabs, eps=1e-12, batch_major=True)
+    np.testing.assert_array_equal(host(bm), host(got).transpose(1, 0, 2))
+    np.testing.assert_array_equal(host(bmidx), wmidx)
+    # ids outside their tables contribute zero rows and raise the flag
+    bad_ids, bad_seg = ids.copy(), seg.copy()
+    bad_ids[3, 2], bad_ids[10, 0], bad_seg[5, 5] = V + 7, -1, 2
+    got, _ = ops.emb_layer_norm(dev(bad_ids), dev(bad_seg), dev(msk), *tabs, eps=1e-12, oob_flag=flag)
+    want, _, n_oob = oracle.emb_layer_norm(bad_ids, bad_seg, msk, word, pos, tok, g, b, eps=1e-12)
+    assert n_oob == 3 and flag.item() == 1
+    assert_close(host(got), want, dtype)
+
+
+@pytest.mark.parametrize("dtype,hidden", [(np.float16, 1024), (np.float32, 1024), (np.float16, 768), (np.float16, 100),
+                                          (np.float16, 128), (np.float32, 64)])
 def test_fused_emb_skip_equals_two_launches(oracle, dtype, hidden):
     """One pass computing LN2(LN(word+pos+tok) + residual + bias) is bit-identical to the
     EmbLayerNorm launch followed by the SkipLayerNorm launch (hidden=100 takes the fallback)."""

@@ -167,6 +167,23 @@ def test_plugin_layer_norm_with_weights_reference_shape(oracle, kats):
     np.testing.assert_array_equal(out, again)
 
 
+def test_plugin_layer_norm_without_weights_reference_shape(oracle):
+    """test_torch_nodes.h:285-291 (layer_norm.pth: torch.layer_norm(x, x.shape[1:], None, None, 1e-5) on
+    [3,3,14,32]): the normalised axes are flattened to one row of 1344 elements, gamma 1 and beta 0."""
+    x = np.random.Generator(np.random.PCG64(14)).standard_normal((3, 3, 14, 32)).astype(np.float32)
+    ld = 3 * 14 * 32
+    c = REG.getPluginCreator("ForwardLayerNormPluginDynamic", "1")
+    p = c.createPlugin("layer_norm", [F("ld", ld), F("beta", np.zeros(ld, np.float32)),
+                                      F("gamma", np.ones(ld, np.float32)), F("type_id", lib.F32),
+                                      F("eps", np.array([1e-5], np.float32))])
+    out = host(p(dev(x.reshape(3, ld)))).reshape(x.shape)
+    ref = torch.nn.functional.layer_norm(torch.from_numpy(x), (3, 14, 32), None, None, 1e-5).numpy()
+    np.testing.assert_allclose(out, ref, atol=1e-3)                      # the reference test's threshold
+    np.testing.assert_allclose(out, ref, rtol=1e-5, atol=1e-5)
+    assert_close(out.reshape(3, ld), oracle.layer_norm(x.reshape(3, ld), np.ones(ld, np.float32),
+                                                       np.zeros(ld, np.float32), eps=1e-5), np.float32)
+
+
 def test_plugins_config5_chain(oracle):
     wl = workloads.config5(variant=1, batch=4, seq=64)
     up = lambda a: a.astype(np.float32)

@@ -237,6 +237,12 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
             ex["config5_fused_emb_skip_layer_norm"] = {
                 "tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
                 "algorithmic_GBs": (wl.emb_algorithmic_bytes() + wl.skip_algorithmic_bytes() - 2 * h2) / (ms * 1e-3) / 1e9}
+    # config 1 (64 bags, the reference's own unit-test shape): one launch's fixed cost, no roofline
+    wl = workloads.config1()
+    tb, ix, of = dev(wl.table), dev(wl.indices), dev(wl.offsets)
+    out = torch.empty((wl.n_bags, wl.table.shape[1]), dtype=tb.dtype, device="cuda")
+    ms = time_graph(torch, lambda: ops.embedding_bag(tb, ix, of, "sum", out=out))
+    ex["config1_sum_fp32_int64"] = {"bags_per_s": wl.n_bags / (ms * 1e-3), "ms": ms}
     for tdt, tname in ((np.float32, "fp32"), (np.float16, "fp16")):
         wl = workloads.config2(table_dtype=tdt)
         tb, ix, of = dev(wl.table), dev(wl.indices), dev(wl.offsets)

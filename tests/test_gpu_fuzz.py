@@ -130,3 +130,40 @@ def test_random_layer_norm_shapes(oracle, seed):
     want = oracle.skip_layer_norm(x, g, b, skip=sk, bias=bi, eps=eps)
     assert got.dtype == dt and got.shape == x.shape
     assert_close(got, want, dt, scale=4.0)
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_table_groups(oracle, seed):
+    """The multi-table launch through ``ops.embedding_bag_group`` on random groups (table count, row
+    width, types, mode, weights on some tables, trailing end offsets, XCD affinity on / off): every
+    column block bit-identical to the oracle's result for that table alone."""
+    r = np.random.Generator(np.random.PCG64(3000 + seed))
+    n_tables = int(r.choice([1, 2, 5, 9, 30, 61]))
+    dim = int(r.choice([4, 8, 32, 64, 128, 200]))
+    tdt = r.choice([np.float32, np.float16])
+    idt = r.choice([np.int32, np.int64])
+    n_bags = int(r.choice([1, 17, 300, 2000]))
+    mode = MODES[int(r.integers(0, 4))]
+    include_last = bool(r.random() < 0.4)
+    weighted = mode == "sum" and r.random() < 0.4
+    tables, ids, offs, psw = [], [], [], []
+    for t in range(n_tables):
+        rows = int(r.choice([1, 3, 50, 700, 9000]))
+        tables.append((r.standard_normal((rows, dim)) * 0.5).astype(tdt))
+        lengths = r.integers(0, int(r.choice([2, 6, 40])), n_bags)
+        n = int(lengths.sum())
+        off = np.concatenate([[0], np.cumsum(lengths)])
+        offs.append((off if include_last else off[:-1]).astype(idt))
+        ids.append(r.integers(0, rows, n).astype(idt))
+        psw.append(r.random(n).astype(tdt) if weighted and r.random() < 0.7 else None)
+    odt = tdt if r.random() < 0.7 else (np.float16 if tdt == np.float32 else np.float32)
+    tt = torch.float16 if odt == np.float16 else torch.float32
+    got = host(ops.embedding_bag_group([dev(t) for t in tables], [dev(i) for i in ids], [dev(o) for o in offs], mode,
+                                       include_last_offset=include_last, out_dtype=tt,
+                                       xcd_table_affinity=bool(seed % 2),
+                                       per_sample_weights=[dev(w) for w in psw] if weighted else None))
+    assert got.shape == (n_bags, n_tables * dim)
+    for t in range(n_tables):
+        want, _, _ = oracle.embedding_bag(tables[t], ids[t], offs[t], ORACLE_OP[mode], per_sample_weights=psw[t],
+                                          include_last_offset=include_last, out_dtype=odt)
+        assert_bits_equal(got[:, t * dim:(t + 1) * dim], want, "seed %d table %d of %d (%s)" % (seed, t, n_tables, mode))

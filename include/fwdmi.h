@@ -135,13 +135,15 @@ int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t of
  * One table of a multi-table batch.  The array of these lives in DEVICE memory.
  */
 typedef struct fwdmi_bag_table {
-  const void* data;    /* [count, dim], 16-byte aligned */
+  const void* data;    /* [count, dim], 16-byte aligned when dim * element size is a multiple of 16 */
   const void* input;   /* [input_size] ids */
   const void* input_2; /* [n_bags] offsets (+1 with include_last_offset) */
   int64_t count;
   int64_t input_size;
   int64_t data_offset;
-  int64_t out_col;     /* first output column of this table's block (a multiple of 8) */
+  int64_t out_col;     /* first output column of this table's block (t * dim for a plain
+                          concatenation); with dim a multiple of 16 bytes of elements it must be
+                          one too */
   const void* weights; /* [input_size] per-sample weights, table dtype; read only with
                           FWDMI_BAG_TABLE_WEIGHTS; may be NULL */
 } fwdmi_bag_table;

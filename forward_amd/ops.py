@@ -150,6 +150,8 @@ class MultiTableBatch:
             _require(self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype,
                      'self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype')
             _require(self.offsets[t].numel() == self.n_bags, 'self.offsets[t].numel() == self.n_bags')
+            _require((self.dim * self.tables[t].element_size()) % 16 != 0 or self.tables[t].data_ptr() % 16 == 0,
+                     'tables of 16-byte-sliceable rows start on a 16-byte boundary')
             w = self.weights[t]
             _require(w is None or (w.dtype == self.tables[t].dtype and w.numel() == self.indices[t].numel()),
                      'per_sample_weights[t] has the table dtype and one entry per id')
@@ -214,6 +216,8 @@ def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offse
                      'per_sample_weights[t] has the table dtype and one entry per id')
             desc[t, 7] = w.data_ptr()
         _require(tab.dim() == 2 and tab.shape[1] == dim and tab.dtype == tdt, 'tables share dim and dtype')
+        _require((dim * tab.element_size()) % 16 != 0 or tab.data_ptr() % 16 == 0,
+                 'tables of 16-byte-sliceable rows start on a 16-byte boundary')
         _require(ids.dim() == 1 and ids.dtype == idt and off.dtype == idt, 'ids are 1-D; ids and offsets share a dtype')
         _require(off.numel() == n_off, 'every table has the same number of offsets')
         desc[t, :7] = (tab.data_ptr(), ids.data_ptr(), off.data_ptr(), tab.shape[0], ids.numel(), 0, t * dim)

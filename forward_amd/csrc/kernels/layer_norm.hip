@@ -660,9 +660,24 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
       FWDMI_HIP_CHECK(hipGetLastError());
       return FWDMI_OK;
     }
-    // Rows that cannot be cut into 16-byte slices (odd length or unaligned operands) are still read
-    // once, one element per lane per slice: a wavefront per row up to 512 elements, a workgroup
-    // per row up to 8192.
+    if (!sliceable && L.ld > 64 * 8 && L.ld <= kWG * 32) {
+      const dim3 bgrid((unsigned)std::max<int64_t>(1, std::min(L.rows, (int64_t)cus * 8)));
+      if (L.ld <= kWG * 4)
+        hipLaunchKernelGGL((ln_block_kernel<T, 1, 4, MODE>), bgrid, block, 0, stream, L);
+      else if (L.ld <= kWG * 8)
+        hipLaunchKernelGGL((ln_block_kernel<T, 1, 8, MODE>), bgrid, block, 0, stream, L);
+      else if (L.ld <= kWG * 16)
+        hipLaunchKernelGGL((ln_block_kernel<T, 1, 16, MODE>), bgrid, block, 0, stream, L);
+      else
+        hipLaunchKernelGGL((ln_block_kernel<T, 1, 32, MODE>), bgrid, block, 0, stream, L);
+      FWDMI_HIP_CHECK(hipGetLastError());
+      return FWDMI_OK;
+    }
+  }
+  // Rows that cannot be cut into 16-byte slices (odd length or unaligned operands) are still read
+  // once, one element per lane per slice: a wavefront per row up to 512 elements (here, embedding
+  // rows included), a workgroup per row up to 8192 (above).
+  if constexpr (MODE != kEmbSkip) {
     if (!sliceable && L.ld <= 64 * 8) {
       const int nv1 = L.ld <= 64 ? 1 : L.ld <= 128 ? 2 : L.ld <= 256 ? 4 : 8;
       if (nv1 == 1)
@@ -673,19 +688,6 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
         hipLaunchKernelGGL((ln_rows_kernel<T, 1, 4, MODE, false>), grid, block, 0, stream, L);
       else
         hipLaunchKernelGGL((ln_rows_kernel<T, 1, 8, MODE, false>), grid, block, 0, stream, L);
-      FWDMI_HIP_CHECK(hipGetLastError());
-      return FWDMI_OK;
-    }
-    if (!sliceable && L.ld <= kWG * 32) {
-      const dim3 bgrid((unsigned)std::max<int64_t>(1, std::min(L.rows, (int64_t)cus * 8)));
-      if (L.ld <= kWG * 4)
-        hipLaunchKernelGGL((ln_block_kernel<T, 1, 4, MODE>), bgrid, block, 0, stream, L);
-      else if (L.ld <= kWG * 8)
-        hipLaunchKernelGGL((ln_block_kernel<T, 1, 8, MODE>), bgrid, block, 0, stream, L);
-      else if (L.ld <= kWG * 16)
-        hipLaunchKernelGGL((ln_block_kernel<T, 1, 16, MODE>), bgrid, block, 0, stream, L);
-      else
-        hipLaunchKernelGGL((ln_block_kernel<T, 1, 32, MODE>), bgrid, block, 0, stream, L);
       FWDMI_HIP_CHECK(hipGetLastError());
       return FWDMI_OK;
     }

@@ -9,9 +9,10 @@
 //
 // Rows of at most 512 bytes share a wavefront (64/G rows at a time, G lanes each); rows too long
 // for one wavefront's registers take a workgroup per row, and so do rows whose length or
-// alignment rule out 128-bit access (one element per lane per slice).  What is left (rows beyond
-// a workgroup's registers, embedding rows without 128-bit access) takes the strided kernel: same
-// reduction, one element per lane per step, row read twice (the second time from cache).
+// alignment rule out 128-bit access and do not fit a wavefront (one element per lane per slice).
+// What is left (rows beyond a workgroup's registers, embedding rows of more than 512 elements
+// without 128-bit access) takes the strided kernel: same reduction, one element per lane per
+// step, row read twice (the second time from cache).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>

@@ -19,6 +19,7 @@ import time
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
+MI355X_PEAK_CLOCK_HZ = 2.4e9    # published peak engine clock
 ROOT = os.path.dirname(os.path.abspath(__file__))
 
 
@@ -385,6 +386,11 @@ def main():
         if result["roofline"]["traffic"]:
             # bytes that crossed the L2 boundary (rocprofv3 counters of the same launch) over this run's time
             result["roofline"]["traffic_GBs"] = result["roofline"]["traffic"] / (ev_ms * 1e-3) / 1e9
+    # the same algorithmic bytes against what the vector L1s can return (64 B per clock and CU): the
+    # unit the row bytes pass through when, as here, most of them hit in cache
+    l1_peak = torch.cuda.get_device_properties(0).multi_processor_count * 64.0 * MI355X_PEAK_CLOCK_HZ / 1e9
+    result["roofline"]["l1_peak_GBs"] = l1_peak
+    result["roofline"]["l1_frac"] = achieved / l1_peak
 
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()

@@ -26,6 +26,8 @@ std::string check_spec(const EmbeddingBagGroupSpec& s) {
   if (!is_float_dtype(s.opt.table_dtype) || !is_float_dtype(s.opt.out_dtype) || !is_index_dtype(s.opt.index_dtype))
     return "unsupported table / index / output type";
   if ((int64_t)T * s.dim > INT32_MAX) return "output row too wide";
+  // at most 2^41 rows of at most 2^24 elements: the byte count must stay far inside 64 bits
+  if (s.total_rows() > ((size_t)1 << 48) / ((size_t)s.dim * 4)) return "tables too large";
   if (s.opt.per_sample_weights && s.op != ReduceOperation::SUM) return "per_sample_weights requires op 0 (sum)";
   return "";
 }

@@ -178,6 +178,13 @@ def test_embedding_bag_group_host_contract(tmp_path):
         c.createPlugin("x", group_fields(tables, extra=[F("max_norm", 1)]))
     with pytest.raises(lib.FwdmiError, match="requires op 0"):
         c.createPlugin("x", group_fields(tables, op=2, extra=[F("per_sample_weights", 1)]))
+    # a blob whose table sizes would wrap 64 bits when multiplied out is refused, not trusted
+    T = 127
+    crafted = struct.pack("<9i", 1 << 24, 0, T, lib.F32, lib.I32, lib.F32, 0, 1, 0) + \
+        struct.pack("<%di" % T, *([2 ** 31 - 1] * T)) + struct.pack("<%di" % T, *([0] * T)) + \
+        struct.pack("<%df" % T, *([1.0] * T)) + struct.pack("<Q", 0)
+    with pytest.raises(lib.FwdmiError, match="too large"):
+        c.deserializePlugin("x", crafted)
     # per-sample weights: a third input per table, in the table's type
     w = c.createPlugin("x", group_fields(tables, extra=[F("per_sample_weights", 1)]))
     wshapes = [(11,), (4,), (11,), (0,), (4,), (0,), (9,), (4,), (9,)]

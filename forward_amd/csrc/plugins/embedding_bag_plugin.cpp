@@ -220,7 +220,7 @@ EmbeddingBagPlugin* EmbeddingBagPlugin::deserialize(const void* data, size_t len
     set_error(FWDMI_ERR_TRUNCATED, "EmbeddingBag: serialized header truncated or malformed");
     return nullptr;
   }
-  if (dim <= 0 || count <= 0 || !is_reduce_op(op)) {
+  if (dim <= 0 || dim > (1 << 24) || count <= 0 || !is_reduce_op(op)) {  // dim: what the launchers accept
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: serialized fields inconsistent (dim %d, count %d, op %d)", dim, count, op);
     return nullptr;
   }
@@ -384,7 +384,7 @@ IPluginV2DynamicExt* EmbeddingBagPluginCreator::createPlugin(const char*, const 
       set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: missing field '%s'", mPluginAttributes[i].name);
       return nullptr;
     }
-  if (dim <= 0 || count <= 0 || !is_reduce_op(op) || !is_index_dtype(opt.index_dtype)) {
+  if (dim <= 0 || dim > (1 << 24) || count <= 0 || !is_reduce_op(op) || !is_index_dtype(opt.index_dtype)) {
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: bad field values (dim %d, count %d, op %d, index_type %d)", dim,
               count, op, opt.index_dtype);
     return nullptr;

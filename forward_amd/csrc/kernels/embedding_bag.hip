@@ -52,17 +52,19 @@ constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting 
 #endif
 // argmax tracking and weights carry more live registers: they keep the looser budget
 #define FWDMI_BAG_OCCUPANCY \
-  __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kWeighted) ? 4 : FWDMI_BAG_WAVES_PER_EU)))
+  __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kWeighted || KIND == kSumSq) ? 4 : FWDMI_BAG_WAVES_PER_EU)))
 constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 
 // kMax also tracks the argmax (needs max_indices); kMaxValue is the plugin's case: values only
-enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3, kMaxValue = 4 };
+// kSumSq: the sum and the sum of squares of the same rows in one pass (two outputs)
+enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3, kMaxValue = 4, kSumSq = 5 };
 
 struct BagLaunch {
   const fwdmi_bag_table* tables;  // device array, or nullptr -> `single`
   fwdmi_bag_table single;
   const void* psw;  // per-sample weights of the single-table form (a table of a batch carries its own)
   void* out;
+  void* out2;  // kSumSq: the sums of squares, laid out like `out`
   void* max_indices;
   int32_t* oob_flag;
   int64_t n_bags;
@@ -246,10 +248,13 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     const bool in_lds = staged && start >= span0 && end <= span0 + span;
 
     float acc[VEC];
+    float acc2[KIND == kSumSq ? VEC : 1];
     constexpr bool kIsMax = KIND == kMax || KIND == kMaxValue;
     TI arg[KIND == kMax ? VEC : 1];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < (KIND == kSumSq ? VEC : 1); ++e) acc2[e] = 0.0f;
 #pragma unroll
     for (int e = 0; e < (KIND == kMax ? VEC : 1); ++e) arg[e] = 0;
     bool first = true;
@@ -362,6 +367,9 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
             acc[e] = __builtin_fmaf(x, one, acc[e]);
           } else if (KIND == kSquare) {
             acc[e] = __builtin_fmaf(x, x, acc[e]);
+          } else if (KIND == kSumSq) {
+            acc[e] = __builtin_fmaf(x, one, acc[e]);
+            acc2[KIND == kSumSq ? e : 0] = __builtin_fmaf(x, x, acc2[KIND == kSumSq ? e : 0]);
           } else if (KIND == kWeighted) {
             acc[e] = __builtin_fmaf(w[u], x, acc[e]);
           } else {
@@ -556,6 +564,31 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
           for (int e = 0; e < VEC; ++e) op[e] = acc[e];
         }
       }
+      if (KIND == kSumSq) {  // second output, same place in its own matrix
+        if (L.out_f16) {
+          _Float16 FWDMI_GLOBAL* op = gmut<_Float16>(L.out2) + o;
+          if (L.vec_store) {
+            Pack<_Float16, VEC> r;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r.v[e] = (_Float16)acc2[KIND == kSumSq ? e : 0];
+            gstore<_Float16, VEC>(op, r);
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) op[e] = (_Float16)acc2[KIND == kSumSq ? e : 0];
+          }
+        } else {
+          float FWDMI_GLOBAL* op = gmut<float>(L.out2) + o;
+          if (L.vec_store) {
+            Pack<float, VEC> r;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r.v[e] = acc2[KIND == kSumSq ? e : 0];
+            gstore<float, VEC>(op, r);
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) op[e] = acc2[KIND == kSumSq ? e : 0];
+          }
+        }
+      }
       if (KIND == kMax && L.max_indices) {
         TI FWDMI_GLOBAL* mp = gmut<TI>(L.max_indices) + (bag0 + lb) * (int64_t)L.dim + col;
 #pragma unroll
@@ -608,6 +641,9 @@ int launch_kind(int kind, const BagLaunch& L, const BagShape& sh, hipStream_t st
     case kSquare:
       hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSquare>), grid, block, sh.lds, stream, L);
       break;
+    case kSumSq:
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSumSq>), grid, block, sh.lds, stream, L);
+      break;
     case kWeighted:
       hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kWeighted>), grid, block, sh.lds, stream, L);
       break;
@@ -651,7 +687,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                  void* output, int64_t n_bags, int64_t fixed_len, int dim, int op, double avg_len,
                  const fwdmi_bag_ext* ext, hipStream_t stream) {
   clear_error();
-  static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0};
+  static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr};
   const fwdmi_bag_ext& x = ext ? *ext : kDefaultExt;
 
   if (!is_float_dtype(x.table_dtype) || !is_float_dtype(x.out_dtype) || !is_index_dtype(x.index_dtype))
@@ -690,6 +726,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   L.single = single;
   L.out = output;
   L.max_indices = x.max_indices;
+  L.out2 = x.square_sum_out;
   L.oob_flag = x.oob_flag;
   L.n_bags = n_bags;
   L.out_stride = out_stride;
@@ -733,13 +770,18 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   L.wgs_per_table = (int)wgs;
   const size_t store_align = std::min<size_t>(16, VEC * so);
   L.vec_store = VEC > 1 && (reinterpret_cast<uintptr_t>(output) % store_align) == 0 &&
+                (reinterpret_cast<uintptr_t>(x.square_sum_out) % store_align) == 0 &&
                 ((out_stride * so) % store_align) == 0 &&
                 (tables_dev || (single.out_col * so) % store_align == 0);
 
   const bool weighted = x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS));
+  FWDMI_REQUIRE(!x.square_sum_out || (op == FWDMI_OP_SUM && !weighted),
+                "embedding bag: square_sum_out needs op SUM without per-sample weights");
   const int kind = op == FWDMI_OP_MAX      ? (x.max_indices ? kMax : kMaxValue)
                    : op == FWDMI_OP_SQUARE_SUM ? kSquare
-                                               : (weighted ? kWeighted : kPlain);
+                   : weighted                  ? kWeighted
+                   : x.square_sum_out          ? kSumSq
+                                               : kPlain;
   L.psw = x.per_sample_weights;
   int grid = (int)(wgs * n_tables);
   L.total_wgs = grid;
@@ -817,9 +859,10 @@ int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t of
     return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "gather: batch %lld x %lld", (long long)batch_size,
                             (long long)offset);
   // A gather is a sum over bags of exactly one id.
-  fwdmi_bag_ext x = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0};
+  fwdmi_bag_ext x = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr};
   x.per_sample_weights = nullptr;
   x.max_indices = nullptr;
+  x.square_sum_out = nullptr;
   x.out_row_stride = 0;
   const int64_t n = batch_size * offset;
   fwdmi_bag_table t{data, input, nullptr, count, n, data_offset, 0, nullptr};

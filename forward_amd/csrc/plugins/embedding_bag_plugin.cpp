@@ -9,7 +9,7 @@ namespace {
 
 bool is_reduce_op(int v) { return v == 0 || v == 1 || v == 2 || v == 3 || v == 999; }
 
-const fwdmi_bag_ext make_ext(const EmbeddingBagOptions& o, const void* psw, int32_t* oob) {
+const fwdmi_bag_ext make_ext(const EmbeddingBagOptions& o, const void* psw, int32_t* oob, void* square_out = nullptr) {
   fwdmi_bag_ext x{};
   x.table_dtype = o.table_dtype;
   x.index_dtype = o.index_dtype;
@@ -20,6 +20,7 @@ const fwdmi_bag_ext make_ext(const EmbeddingBagOptions& o, const void* psw, int3
   x.out_row_stride = 0;
   x.oob_flag = oob;
   x.flags = 0;
+  x.square_sum_out = square_out;
   return x;
 }
 
@@ -32,8 +33,8 @@ EmbeddingBagPlugin::EmbeddingBagPlugin(std::shared_ptr<HostDeviceBlob> table, in
 
 EmbeddingBagPlugin::~EmbeddingBagPlugin() noexcept { terminate(); }
 
-// One output: the reduced bags (embedding_bag_plugin.cpp:55).
-int EmbeddingBagPlugin::getNbOutputs() const noexcept { return 1; }
+// One output: the reduced bags (embedding_bag_plugin.cpp:55); "002" with with_square_sum: two.
+int EmbeddingBagPlugin::getNbOutputs() const noexcept { return opt_.with_square_sum ? 2 : 1; }
 
 // Shape rules of embedding_bag_plugin.cpp:57-100.
 //   1 input  [B, L]           -> [B, dim]            (reduce)
@@ -41,7 +42,8 @@ int EmbeddingBagPlugin::getNbOutputs() const noexcept { return 1; }
 //   2 inputs ids [N], offsets [B] or [1, B] -> [B, dim]   (GATHER not allowed)
 Dims EmbeddingBagPlugin::getOutputDimensions(int outputIndex, const Dims* inputs, int nbInputs) noexcept {
   clear_error();
-  if (outputIndex != 0 || !inputs || nbInputs < 1 || nbInputs > (opt_.per_sample_weights ? 3 : 2)) {
+  if (outputIndex < 0 || outputIndex >= getNbOutputs() || !inputs || nbInputs < 1 ||
+      nbInputs > (opt_.per_sample_weights ? 3 : 2)) {
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: output %d with %d inputs", outputIndex, nbInputs);
     return error_dims();
   }
@@ -80,7 +82,8 @@ Dims EmbeddingBagPlugin::getOutputDimensions(int outputIndex, const Dims* inputs
 bool EmbeddingBagPlugin::supportsFormatCombination(int pos, const PluginTensorDesc* inOut, int nbInputs,
                                                    int nbOutputs) noexcept {
   const int max_inputs = opt_.per_sample_weights ? 3 : 2;
-  if (!inOut || nbInputs < 1 || nbInputs > max_inputs || nbOutputs != 1 || pos < 0 || pos >= nbInputs + nbOutputs)
+  if (!inOut || nbInputs < 1 || nbInputs > max_inputs || nbOutputs != getNbOutputs() || pos < 0 ||
+      pos >= nbInputs + nbOutputs)
     return false;
   const PluginTensorDesc& d = inOut[pos];
   if (d.format != FWDMI_FORMAT_LINEAR) return false;
@@ -140,7 +143,7 @@ int EmbeddingBagPlugin::enqueue(const PluginTensorDesc* inputDesc, const PluginT
     return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag::enqueue: ids must be 1-D or 2-D, got %d-D", in0.nbDims);
   if (in0.nbDims > 1) {
     const int64_t batch_size = in0.d[0], bag_len = in0.d[1];
-    const fwdmi_bag_ext x = make_ext(opt_, nullptr, d_oob_);
+    const fwdmi_bag_ext x = make_ext(opt_, nullptr, d_oob_, opt_.with_square_sum ? outputs[1] : nullptr);
     if (op_ == ReduceOperation::GATHER)
       return fwdmi_gather(inputs[0], outputs[0], batch_size, bag_len, d_data_, count_, dim_, data_offset_, &x,
                           hipStream);
@@ -155,7 +158,8 @@ int EmbeddingBagPlugin::enqueue(const PluginTensorDesc* inputDesc, const PluginT
     return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag::enqueue: offsets must be [B] or [1, B]");
   const int64_t n_off = in1.nbDims == 1 ? in1.d[0] : in1.d[1];
   const int64_t n_bags = n_off - (opt_.include_last_offset ? 1 : 0);
-  const fwdmi_bag_ext x = make_ext(opt_, opt_.per_sample_weights ? inputs[2] : nullptr, d_oob_);
+  const fwdmi_bag_ext x = make_ext(opt_, opt_.per_sample_weights ? inputs[2] : nullptr, d_oob_,
+                                   opt_.with_square_sum ? outputs[1] : nullptr);
   return fwdmi_embedding_bag(inputs[0], inputs[1], outputs[0], input_size, n_bags, d_data_, count_, dim_,
                              data_offset_, static_cast<int>(op_), &x, hipStream);
 }
@@ -164,12 +168,13 @@ int EmbeddingBagPlugin::enqueue(const PluginTensorDesc* inputDesc, const PluginT
 //   int dim | int count | int data_offset | int op | size_t n | float[n]
 // "002" bytes:
 //   int dim | int count | int data_offset | int op | int table_dtype | int index_dtype |
-//   int out_dtype | int include_last_offset | int per_sample_weights | size_t n | elem[n]
+//   int out_dtype | int include_last_offset | int per_sample_weights | int with_square_sum |
+//   size_t n | elem[n]
 // A "002" plugin whose table was given by file (`data_file`) writes, in place of the table,
 //   size_t SIZE_MAX | size_t path_len | path bytes | uint64 byte offset in the file
 // so an engine file stays small and loading maps the table instead of copying it.
 size_t EmbeddingBagPlugin::getSerializationSize() const noexcept {
-  const size_t head = 4 * sizeof(int) + (version_ext_ ? 5 * sizeof(int) : 0) + sizeof(size_t);
+  const size_t head = 4 * sizeof(int) + (version_ext_ ? 6 * sizeof(int) : 0) + sizeof(size_t);
   if (table_->by_reference()) return head + sizeof(size_t) + table_->path().size() + sizeof(uint64_t);
   return head + table_->size();
 }
@@ -186,6 +191,7 @@ void EmbeddingBagPlugin::serialize(void* buffer) const noexcept {
     w.pod<int>(opt_.out_dtype);
     w.pod<int>(opt_.include_last_offset);
     w.pod<int>(opt_.per_sample_weights);
+    w.pod<int>(opt_.with_square_sum);
   }
   if (table_->by_reference()) {
     w.pod<size_t>(SIZE_MAX);
@@ -214,13 +220,15 @@ EmbeddingBagPlugin* EmbeddingBagPlugin::deserialize(const void* data, size_t len
     r.pod(&opt.out_dtype);
     r.pod(&opt.include_last_offset);
     r.pod(&opt.per_sample_weights);
+    r.pod(&opt.with_square_sum);
   }
   if (!r.ok() || !is_float_dtype(opt.table_dtype) || !is_float_dtype(opt.out_dtype) ||
       !is_index_dtype(opt.index_dtype)) {
     set_error(FWDMI_ERR_TRUNCATED, "EmbeddingBag: serialized header truncated or malformed");
     return nullptr;
   }
-  if (dim <= 0 || dim > (1 << 24) || count <= 0 || !is_reduce_op(op)) {  // dim: what the launchers accept
+  if (dim <= 0 || dim > (1 << 24) || count <= 0 || !is_reduce_op(op) ||  // dim: what the launchers accept
+      (opt.with_square_sum && (op != FWDMI_OP_SUM || opt.per_sample_weights))) {
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: serialized fields inconsistent (dim %d, count %d, op %d)", dim, count, op);
     return nullptr;
   }
@@ -300,6 +308,7 @@ EmbeddingBagPluginCreator::EmbeddingBagPluginCreator(bool version_ext) : version
     declare("output_fp16", PluginFieldType::kINT32);
     declare("include_last_offset", PluginFieldType::kINT32);
     declare("per_sample_weights", PluginFieldType::kINT32);
+    declare("with_square_sum", PluginFieldType::kINT32);
     declare("data_file", PluginFieldType::kCHAR);
     declare("data_file_row_offset", PluginFieldType::kINT32);
     declare("table_type", PluginFieldType::kINT32);
@@ -341,6 +350,7 @@ IPluginV2DynamicExt* EmbeddingBagPluginCreator::createPlugin(const char*, const 
     else if (name == "op") scalar = &op, slot = 3;
     else if (version_ext_ && name == "include_last_offset") scalar = &opt.include_last_offset;
     else if (version_ext_ && name == "per_sample_weights") scalar = &opt.per_sample_weights;
+    else if (version_ext_ && name == "with_square_sum") scalar = &opt.with_square_sum;
     else if (version_ext_ && name == "index_type") scalar = &opt.index_dtype;
     else if (version_ext_ && name == "data_file_row_offset") scalar = &file_row_offset;
     else if (version_ext_ && name == "table_type") scalar = &table_type;
@@ -391,6 +401,10 @@ IPluginV2DynamicExt* EmbeddingBagPluginCreator::createPlugin(const char*, const 
   }
   if (opt.per_sample_weights && op != FWDMI_OP_SUM) {
     set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: per_sample_weights requires op SUM");
+    return nullptr;
+  }
+  if (opt.with_square_sum && (op != FWDMI_OP_SUM || opt.per_sample_weights)) {
+    set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: with_square_sum requires op SUM without per_sample_weights");
     return nullptr;
   }
   const size_t n = (size_t)dim * (size_t)count;

@@ -5,8 +5,9 @@
 // embedding_bag_plugin.cpp:37-300): same creator fields, shape rules, format rules, dispatch
 // and serialized bytes.  Version "001" is the reference contract (fp32 table, int32 ids,
 // fp32 output, exactly five fields).  Version "002" adds optional fields for fp16 tables,
-// int64 ids, fp16 output, include_last_offset and a per-sample-weights input, and appends them
-// to the serialized layout.
+// int64 ids, fp16 output, include_last_offset, a per-sample-weights input and a second output
+// with the sums of squares (the pair a factorisation-machine term needs, from one pass), and
+// appends them to the serialized layout.
 #pragma once
 
 #include <memory>
@@ -29,9 +30,10 @@ struct EmbeddingBagOptions {
   int32_t out_dtype = FWDMI_F32;
   int32_t include_last_offset = 0;
   int32_t per_sample_weights = 0;  // 1: a third input carries per-sample weights
+  int32_t with_square_sum = 0;     // 1 (op SUM): a second output carries the sums of squares
   bool is_default() const {
     return table_dtype == FWDMI_F32 && index_dtype == FWDMI_I32 && out_dtype == FWDMI_F32 &&
-           !include_last_offset && !per_sample_weights;
+           !include_last_offset && !per_sample_weights && !with_square_sum;
   }
 };
 

@@ -31,7 +31,7 @@ class BagExt(C.Structure):
     _fields_ = [("table_dtype", C.c_int32), ("index_dtype", C.c_int32), ("out_dtype", C.c_int32),
                 ("include_last_offset", C.c_int32), ("per_sample_weights", C.c_void_p),
                 ("max_indices", C.c_void_p), ("out_row_stride", C.c_int64), ("oob_flag", C.c_void_p),
-                ("flags", C.c_int32), ("table_cost", C.c_void_p)]
+                ("flags", C.c_int32), ("table_cost", C.c_void_p), ("square_sum_out", C.c_void_p)]
 
 
 class EmbExt(C.Structure):
@@ -41,7 +41,8 @@ class EmbExt(C.Structure):
 
 class BagTable(C.Structure):
     _fields_ = [("data", C.c_void_p), ("input", C.c_void_p), ("input_2", C.c_void_p), ("count", C.c_int64),
-                ("input_size", C.c_int64), ("data_offset", C.c_int64), ("out_col", C.c_int64)]
+                ("input_size", C.c_int64), ("data_offset", C.c_int64), ("out_col", C.c_int64),
+                ("weights", C.c_void_p)]
 
 
 class Dims(C.Structure):

@@ -44,7 +44,7 @@ def _op(mode):
 
 
 def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_indices=None, out_row_stride=0,
-         oob_flag=None, flags=0, table_cost=None):
+         oob_flag=None, flags=0, table_cost=None, square_sum_out=None):
     x = lib.BagExt()
     x.table_dtype = _FDT[table.dtype]
     x.index_dtype = _IDT[indices.dtype]
@@ -56,16 +56,18 @@ def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_ind
     x.oob_flag = oob_flag.data_ptr() if oob_flag is not None else None
     x.flags = flags
     x.table_cost = table_cost.ctypes.data if table_cost is not None else None
+    x.square_sum_out = square_sum_out.data_ptr() if square_sum_out is not None else None
     return x
 
 
 def embedding_bag(table, indices, offsets, mode="sum", per_sample_weights=None, include_last_offset=False,
                   data_offset=0, out_dtype=None, out=None, out_col=0, want_max_indices=False, oob_flag=None,
-                  count=None, stream=None):
+                  count=None, stream=None, with_square_sum=False):
     """Bags over a 1-D ``indices`` + ``offsets`` layout -> ``[n_bags, dim]``.
 
     ``out`` / ``out_col`` write a column block of an existing ``[n_bags, W]`` matrix.
-    Returns ``out`` or ``(out, max_indices)``.
+    Returns ``out`` or ``(out, max_indices)``; with ``with_square_sum`` (mode "sum", no weights)
+    ``(out, square_sums)``: both reductions from one pass over the rows.
     """
     table, indices, offsets = _dev(table, "table"), _dev(indices, "indices"), _dev(offsets, "offsets")
     if indices.dtype != offsets.dtype:
@@ -89,24 +91,33 @@ def embedding_bag(table, indices, offsets, mode="sum", per_sample_weights=None, 
         _require(psw.dtype == table.dtype and psw.numel() == indices.numel(),
                  'psw.dtype == table.dtype and psw.numel() == indices.numel()')
     mi = torch.empty((n_bags, dim), dtype=indices.dtype, device=table.device) if want_max_indices else None
-    x = _ext(table, indices, odt, include_last_offset, psw, mi, stride, oob_flag)
+    sq = None
+    if with_square_sum:
+        _require(stride == 0 and not want_max_indices, 'with_square_sum writes two packed [n_bags, dim] outputs')
+        sq = torch.empty((n_bags, dim), dtype=odt, device=table.device)
+    x = _ext(table, indices, odt, include_last_offset, psw, mi, stride, oob_flag, square_sum_out=sq)
     lib.check(lib.dll.fwdmi_embedding_bag(_p(indices), _p(offsets), _p(dst), indices.numel(), n_bags, _p(table),
                                           table.shape[0] if count is None else count, dim, data_offset, _op(mode),
                                           C.byref(x), _stream(stream)))
+    if with_square_sum:
+        return out, sq
     return (out, mi) if want_max_indices else out
 
 
-def embedding_bag_fixed(table, indices, mode="sum", data_offset=0, out_dtype=None, oob_flag=None, stream=None):
-    """Fixed-length bags: ``indices`` is ``[B, L]`` -> ``[B, dim]``."""
+def embedding_bag_fixed(table, indices, mode="sum", data_offset=0, out_dtype=None, oob_flag=None, stream=None,
+                        with_square_sum=False):
+    """Fixed-length bags: ``indices`` is ``[B, L]`` -> ``[B, dim]`` (``with_square_sum``: also the
+    sums of squares, from the same pass)."""
     table, indices = _dev(table, "table"), _dev(indices, "indices")
     _require(indices.dim() == 2, 'indices.dim() == 2')
     b, l = indices.shape
     odt = table.dtype if out_dtype is None else out_dtype
     out = torch.empty((b, table.shape[1]), dtype=odt, device=table.device)
-    x = _ext(table, indices, odt, oob_flag=oob_flag)
+    sq = torch.empty_like(out) if with_square_sum else None
+    x = _ext(table, indices, odt, oob_flag=oob_flag, square_sum_out=sq)
     lib.check(lib.dll.fwdmi_embedding_bag_fixed(_p(indices), _p(out), b, l, _p(table), table.shape[0], table.shape[1],
                                                 data_offset, _op(mode), C.byref(x), _stream(stream)))
-    return out
+    return (out, sq) if with_square_sum else out
 
 
 def gather(table, indices, data_offset=0, out_dtype=None, oob_flag=None, stream=None):

@@ -89,6 +89,12 @@ typedef struct fwdmi_bag_ext {
   int32_t flags;               /* FWDMI_BAG_* bits, 0 for none */
   const float* table_cost;     /* HOST array [n_tables] or NULL: relative cost of one bag of each
                                   table, used by FWDMI_BAG_XCD_TABLE_AFFINITY */
+  void* square_sum_out;        /* device, out dtype, laid out like the output (same row stride and
+                                  column blocks); op SUM without weights only; may be NULL.  When
+                                  given, the same pass also writes the sum of squares of every
+                                  bag: the two reductions a factorisation-machine term needs
+                                  (the reference builds them as two plugins over two copies of
+                                  the table, source/fwd_tf/tf_cvt/tf_desc_creators/tf_embedding_bag_creator.h:43-95) */
 } fwdmi_bag_ext;
 
 /* Multi-table launches only: renumber workgroups so that each of the 8 XCDs (one L2 each)

@@ -421,3 +421,42 @@ def test_concurrent_enqueue_from_threads_on_their_own_streams(oracle):
     for k in range(4):
         for got in results[k]:
             assert_bits_equal(got, want, "thread %d" % k)
+
+
+@pytest.mark.parametrize("tdt,idt", [(np.float32, np.int32), (np.float16, np.int64), (np.float16, np.int32)])
+def test_sum_and_square_sum_in_one_pass(oracle, tdt, idt):
+    """The two reductions of a factorisation-machine term (the reference builds them as two plugins,
+    op 0 and op 3, over the same ids): one pass writes both, each bit-identical to its own launch."""
+    rng = np.random.Generator(np.random.PCG64(55))
+    for dim in (8, 64, 100, 128, 520):
+        table = (rng.standard_normal((3000, dim)) * 0.5).astype(tdt)
+        ids2d = rng.integers(-2, 3002, (400, 13)).astype(idt)            # a few ids outside the table
+        s, q = ops.embedding_bag_fixed(dev(table), dev(ids2d), "sum", with_square_sum=True)
+        ws, _, _ = oracle.embedding_bag(table, ids2d, None, oracle.OP_SUM)
+        wq, _, _ = oracle.embedding_bag(table, ids2d, None, oracle.OP_SQUARE_SUM)
+        assert_bits_equal(host(s), ws, "sums, dim %d" % dim)
+        assert_bits_equal(host(q), wq, "sums of squares, dim %d" % dim)
+        lengths = rng.integers(0, 30, 500)
+        off = np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(idt)
+        ids = rng.integers(0, 3000, int(lengths.sum())).astype(idt)
+        s, q = ops.embedding_bag(dev(table), dev(ids), dev(off), "sum", with_square_sum=True, out_dtype=torch.float32)
+        ws, _, _ = oracle.embedding_bag(table, ids, off, oracle.OP_SUM, out_dtype=np.float32)
+        wq, _, _ = oracle.embedding_bag(table, ids, off, oracle.OP_SQUARE_SUM, out_dtype=np.float32)
+        assert_bits_equal(host(s), ws, "offsets form, sums, dim %d" % dim)
+        assert_bits_equal(host(q), wq, "offsets form, sums of squares, dim %d" % dim)
+    with pytest.raises(lib.FwdmiError, match="square_sum_out"):
+        ops.embedding_bag_fixed(dev(table), dev(ids2d), "max", with_square_sum=True)
+
+    # through the plugin: "002" with with_square_sum has two outputs
+    c2 = REG.getPluginCreator("EmbeddingBag_TRT", "002")
+    table = (rng.standard_normal((50, 8)) * 0.5).astype(np.float32)
+    ids2d = rng.integers(0, 50, (10, 5)).astype(np.int32)                # the shape of the reference's TF test
+    p = c2.createPlugin("fm", bag_fields(table) + [F("with_square_sum", 1)])
+    assert p.getNbOutputs() == 2 and p.getOutputDimensions(1, [(10, 5)]) == [10, 8]
+    s, q = p(dev(ids2d))
+    assert_bits_equal(host(s), oracle.embedding_bag(table, ids2d, None, 0)[0], "plugin sums")
+    assert_bits_equal(host(q), oracle.embedding_bag(table, ids2d, None, 3)[0], "plugin sums of squares")
+    s2, q2 = c2.deserializePlugin("fm", p.serialize())(dev(ids2d))
+    assert torch.equal(s, s2) and torch.equal(q, q2)
+    with pytest.raises(lib.FwdmiError, match="with_square_sum"):
+        c2.createPlugin("fm", bag_fields(table, op=3) + [F("with_square_sum", 1)])

@@ -75,14 +75,14 @@ def test_table_by_file_reference_host_side(tmp_path):
     p = c.createPlugin("emb", fields)
     blob = p.serialize()
     assert len(blob) < 200                                   # a reference, not 3200 bytes of table
-    head = struct.unpack("<9iQQ", blob[:52])
-    assert head[:9] == (16, 100, 0, 0, lib.F16, lib.I32, lib.F16, 0, 0) and head[9] == 2**64 - 1 and head[10] == len(tf)
-    assert blob[52:52 + len(tf)] == tf.encode() and struct.unpack("<Q", blob[-8:]) == (10 * 16 * 2,)
+    head = struct.unpack("<10iQQ", blob[:56])
+    assert head[:10] == (16, 100, 0, 0, lib.F16, lib.I32, lib.F16, 0, 0, 0) and head[10] == 2**64 - 1 and head[11] == len(tf)
+    assert blob[56:56 + len(tf)] == tf.encode() and struct.unpack("<Q", blob[-8:]) == (10 * 16 * 2,)
     q = c.deserializePlugin("emb", blob)
     assert q.serialize() == blob and q.clone().serialize() == blob
     # the same table given by value serializes by value
     byval = c.createPlugin("emb", bag_fields(table) + [F("output_fp16", 1)])
-    assert byval.serialize()[44:] == table.tobytes()
+    assert byval.serialize()[48:] == table.tobytes()
     # a file that is too short, a missing file, both 'data' and 'data_file'
     with pytest.raises(lib.FwdmiError, match="shorter"):
         c.createPlugin("emb", fields[:6] + [F("data_file_row_offset", 50)])

@@ -112,8 +112,8 @@ def test_embedding_bag_extended_version():
     assert not p.supportsFormatCombination(0, [((40,), lib.I32)] + io[1:], 3, 1)
     assert p.getOutputDataType(0, [lib.I64, lib.I64, lib.F16]) == lib.F16
     blob = p.serialize()
-    assert struct.unpack("<9iQ", blob[:44]) == (8, 9, 0, 0, lib.F16, lib.I64, lib.F16, 1, 1, 72)
-    assert blob[44:] == table.tobytes()
+    assert struct.unpack("<10iQ", blob[:48]) == (8, 9, 0, 0, lib.F16, lib.I64, lib.F16, 1, 1, 0, 72)
+    assert blob[48:] == table.tobytes()
     assert c.deserializePlugin("e", blob).serialize() == blob
     with pytest.raises(lib.FwdmiError, match="SUM"):
         c.createPlugin("e", bag_fields(table, op=2) + [F("per_sample_weights", 1)])

@@ -273,7 +273,8 @@ typedef struct fwdmi_plugin_field {
 
 /* getPluginRegistry()->getPluginCreator(name, version), trt_embedding_bag_creator.h:54-55.
  * Registered: "EmbeddingBag_TRT"/"001" (the reference contract) and "002" (fp16 tables, int64 ids,
- * fp16 output, include_last_offset, per-sample weights, tables by file reference),
+ * fp16 output, include_last_offset, per-sample weights, a second output with the sums of squares,
+ * tables by file reference),
  * "EmbeddingBagGroup_TRT"/"001" (T tables + their concatenation, one launch per enqueue; needs
  * getWorkspaceSize bytes of workspace), "CustomEmbLayerNormPluginDynamic"/"1",
  * "CustomSkipLayerNormPluginDynamic"/"1", "ForwardLayerNormPluginDynamic"/"1". NULL if absent. */

@@ -10,9 +10,9 @@
 // Rows of at most 512 bytes share a wavefront (64/G rows at a time, G lanes each); rows too long
 // for one wavefront's registers take a workgroup per row, and so do rows whose length or
 // alignment rule out 128-bit access and do not fit a wavefront (one element per lane per slice).
-// What is left (rows beyond a workgroup's registers, embedding rows of more than 512 elements
-// without 128-bit access) takes the strided kernel: same reduction, one element per lane per
-// step, row read twice (the second time from cache).
+// Rows beyond a workgroup's registers are streamed twice by a workgroup (the second time from
+// cache).  What is left (embedding rows of more than 512 elements without 128-bit access) takes
+// the strided kernel: one element per lane per step, row read twice.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -530,6 +530,85 @@ __global__ __launch_bounds__(kWG) void ln_block_kernel(const LnLaunch L) {
   }
 }
 
+// Rows beyond a workgroup's registers: a workgroup per row, two passes over the row in slices of
+// VEC elements per lane.  The first pass accumulates sums of (x - x0) and (x - x0)^2 with x0 the
+// row's first element (the shifted form keeps the cancellation of the one-pass variance small),
+// the second pass re-reads the row (from cache) and writes the result.  kLayerNorm / kSkip only.
+template <typename T, int VEC, int MODE>
+__global__ __launch_bounds__(kWG) void ln_stream_kernel(const LnLaunch L) {
+  __shared__ float s_part[kWavesPerWG][4];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave_in_wg = tid >> 6;
+  const T FWDMI_GLOBAL* const in0 = gconst<T>(L.input);
+  const T FWDMI_GLOBAL* const in1 = gconst<T>(L.skip);
+  const float one = L.one;
+  auto value = [&](int64_t base, int c, float* x) {
+    const Pack<T, VEC> a = gload<T, VEC>(in0 + base + c);
+    Pack<T, VEC> b{};
+    if (MODE == kSkip) b = gload<T, VEC>(in1 + base + c);
+    Pack<float, VEC> pi{};
+    if (L.bias) pi = gload<float, VEC>(gconst<float>(L.bias) + c);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      float v = (float)a.v[e];
+      if (MODE == kSkip) v = __builtin_fmaf((float)b.v[e], one, v);
+      x[e] = v + (L.bias ? pi.v[e] : 0.0f);
+    }
+  };
+  for (int64_t r = blockIdx.x; r < L.rows; r += gridDim.x) {
+    const int64_t base = r * L.ld;
+    float x0;
+    {
+      float v = (float)in0[base];
+      if (MODE == kSkip) v = __builtin_fmaf((float)in1[base], one, v);
+      x0 = v + (L.bias ? L.bias[0] : 0.0f);
+    }
+    float n = 0.0f, s1 = 0.0f, s2 = 0.0f;
+    for (int c = tid * VEC; c < L.ld; c += kWG * VEC) {
+      float x[VEC];
+      value(base, c, x);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float d = x[e] - x0;
+        s1 += d;
+        s2 = __builtin_fmaf(d, d, s2);
+      }
+      n += (float)VEC;
+    }
+    Welford w{n, 0.0f, 0.0f};
+    if (n > 0.0f) {
+      const float inv = 1.0f / n;
+      w.mean = x0 + s1 * inv;
+      w.m2 = fmaxf(s2 - s1 * s1 * inv, 0.0f);
+    }
+    w = wave_allreduce(w);
+    if (lane == 0) {
+      s_part[wave_in_wg][0] = w.n;
+      s_part[wave_in_wg][1] = w.mean;
+      s_part[wave_in_wg][2] = w.m2;
+    }
+    __syncthreads();
+    Welford t{s_part[0][0], s_part[0][1], s_part[0][2]};
+#pragma unroll
+    for (int k = 1; k < kWavesPerWG; ++k) t = merge(t, Welford{s_part[k][0], s_part[k][1], s_part[k][2]});
+    __syncthreads();  // s_part is rewritten for the next row
+    const float mu = t.mean;
+    const float rs = __builtin_amdgcn_rsqf(__builtin_fmaf(t.m2, __builtin_amdgcn_rcpf(t.n), L.eps));
+    T FWDMI_GLOBAL* op = gmut<T>(L.output) + base;
+    for (int c = tid * VEC; c < L.ld; c += kWG * VEC) {
+      float x[VEC];
+      value(base, c, x);
+      const Pack<float, VEC> pg = gload<float, VEC>(gconst<float>(L.gamma) + c);
+      const Pack<float, VEC> pb = gload<float, VEC>(gconst<float>(L.beta) + c);
+      Pack<T, VEC> o;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o.v[e] = round_to<T>(__builtin_fmaf(pg.v[e], (x[e] - mu) * rs, pb.v[e]));
+      gstore<T, VEC>(op + c, o);
+    }
+  }
+}
+
 // Any ld, any alignment: one element per lane per step, two passes over the row.
 template <typename T, int MODE>
 __global__ __launch_bounds__(kWG) void ln_strided_kernel(const LnLaunch L) {
@@ -671,6 +750,19 @@ int ln_launch(LnLaunch& L, bool vec_ok, hipStream_t stream) {
         hipLaunchKernelGGL((ln_block_kernel<T, 1, 16, MODE>), bgrid, block, 0, stream, L);
       else
         hipLaunchKernelGGL((ln_block_kernel<T, 1, 32, MODE>), bgrid, block, 0, stream, L);
+      FWDMI_HIP_CHECK(hipGetLastError());
+      return FWDMI_OK;
+    }
+  }
+  if constexpr (!is_emb(MODE)) {
+    const int block_chunks = (L.ld + kWG * kVec - 1) / (kWG * kVec);
+    if ((sliceable && block_chunks > 8) || (!sliceable && L.ld > kWG * 32)) {
+      // longer than a workgroup's registers hold: two passes, the second from cache
+      const dim3 bgrid((unsigned)std::max<int64_t>(1, std::min(L.rows, (int64_t)cus * 8)));
+      if (sliceable)
+        hipLaunchKernelGGL((ln_stream_kernel<T, kVec, MODE>), bgrid, block, 0, stream, L);
+      else
+        hipLaunchKernelGGL((ln_stream_kernel<T, 1, MODE>), bgrid, block, 0, stream, L);
       FWDMI_HIP_CHECK(hipGetLastError());
       return FWDMI_OK;
     }

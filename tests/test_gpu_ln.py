@@ -71,7 +71,9 @@ def test_config5_emb_then_skip_layer_norm(oracle, dtype):
                                       # a workgroup per row, and beyond it the strided kernel
                                       (4104, np.float16), (12000, np.float16), (16384, np.float16),
                                       (16392, np.float16), (4096, np.float32), (8192, np.float32),
-                                      (8196, np.float32)])
+                                      (8196, np.float32),
+                                      # beyond a workgroup's registers: streamed twice
+                                      (40000, np.float16), (20001, np.float32), (65536, np.float32)])
 def test_layer_norm_row_lengths(oracle, ld, dtype):
     rng = np.random.Generator(np.random.PCG64(ld))
     x = (rng.standard_normal((37, ld)) * 2 + 0.5).astype(dtype)
@@ -88,11 +90,13 @@ def test_layer_norm_row_lengths(oracle, ld, dtype):
     assert_close(got, oracle.skip_layer_norm(x, g, b, skip=sk, bias=bi, eps=eps), dtype)
 
 
-def test_layer_norm_large_mean_is_stable(oracle):
-    """|mean| >> std: the E[x^2]-mean^2 form of the reference loses all digits here; Welford does not."""
+@pytest.mark.parametrize("ld", [1024, 24, 6000, 20000])
+def test_layer_norm_large_mean_is_stable(oracle, ld):
+    """|mean| >> std: the E[x^2]-mean^2 form of the reference loses all digits here; Welford (and, for
+    streamed rows, sums shifted by the row's first element) does not.  One length per kernel variant."""
     rng = np.random.Generator(np.random.PCG64(9))
-    x = (1000.0 + 0.1 * rng.standard_normal((64, 1024))).astype(np.float32)
-    g, b = np.ones(1024, np.float32), np.zeros(1024, np.float32)
+    x = (1000.0 + 0.1 * rng.standard_normal((64, ld))).astype(np.float32)
+    g, b = np.ones(ld, np.float32), np.zeros(ld, np.float32)
     got = host(ops.layer_norm(dev(x), dev(g), dev(b), eps=0.0))
     want = oracle.layer_norm(x, g, b, eps=0.0)
     np.testing.assert_allclose(got, want, rtol=1e-3, atol=1e-3)

@@ -296,7 +296,7 @@ def sweep_layer_norm(torch, ops):
     same GPU, both timed as 10 launches captured in one HIP graph."""
     print("%7s %6s %5s | %9s %8s | %9s | %s" % ("rows", "ld", "type", "ms", "GB/s", "torch ms", "speedup"), flush=True)
     for tdt in (torch.float16, torch.float32):
-        for ld in (64, 128, 256, 768, 1000, 1024, 2048, 4096, 8192):
+        for ld in (64, 128, 256, 768, 1000, 1024, 2048, 4096, 8192, 32768):
             for rows in (1024, 8192, 65536, 262144):
                 if rows * ld * 4 > (1 << 30):
                     continue

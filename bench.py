@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the embedding-side hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config4] [--no-cpu] [--no-extra]
+  python bench.py [--gpus 1] [--steps K (200)] [--warmup W (20)] [--workload config4] [--no-cpu] [--no-extra]
 
 A step is one pass of the DLRM-style sparse stage (BASELINE config 4): 26 sum-mode tables, fp16
 rows of dim 128, 65536 bags per table with truncated-Zipf lengths, Zipf ids, fp16 output
@@ -30,8 +30,8 @@ def log(*a):
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="config4", choices=["config4"])
     ap.add_argument("--tables", type=int, default=26, help="debug only: fewer tables (not the named config)")
     ap.add_argument("--bags", type=int, default=65536, help="debug only: smaller batch (not the named config)")

@@ -21,8 +21,8 @@
 //     part of the table-major work list, cut at equal estimated cost.
 //
 // Memory safety: offsets are clamped to [0, input_size] and made non-decreasing before use,
-// ids outside [data_offset, data_offset+count) never form an address, so arbitrary input
-// bytes cannot make the kernel read or write out of bounds.
+// ids outside [data_offset, data_offset+count) never form an address (a table of no rows forms
+// none at all), so arbitrary id / offset bytes cannot make the kernel read or write out of bounds.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -152,6 +152,29 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   if (tid == 0) s_next = slots;
   for (int i = tid; i < kLenBuckets; i += wg_lanes) s_hist[i] = 0;
   __syncthreads();
+
+  // A table without rows (count <= 0; its data pointer may be null): every id is outside it, so
+  // the run's bags are zeros and no row address is ever formed.  Uniform over the workgroup.
+  if (T.count <= 0) {
+    bool any = false;
+    const int64_t n_el = (int64_t)nb * L.dim;
+    for (int64_t i = tid; i < n_el; i += wg_lanes) {
+      const int lb = (int)(i / L.dim);
+      const int c = (int)(i - (int64_t)lb * L.dim);
+      any |= s_off[lb + 1] > s_off[lb];
+      const int64_t o = (bag0 + lb) * L.out_stride + T.out_col + c;
+      if (L.out_f16) {
+        gmut<_Float16>(L.out)[o] = (_Float16)0.0f;
+        if (KIND == kSumSq) gmut<_Float16>(L.out2)[o] = (_Float16)0.0f;
+      } else {
+        gmut<float>(L.out)[o] = 0.0f;
+        if (KIND == kSumSq) gmut<float>(L.out2)[o] = 0.0f;
+      }
+      if (KIND == kMax && L.max_indices) gmut<TI>(L.max_indices)[(bag0 + lb) * (int64_t)L.dim + c] = 0;
+    }
+    if (any && L.oob_flag) atomicOr(L.oob_flag, 1);
+    return;
+  }
 
   // A "compact" table has at most 2^24 rows and 4 GiB: a row number fits 32 bits (whatever the
   // id type) and a row's byte offset is one 24-bit multiply-add on top of a uniform base.

@@ -466,7 +466,10 @@ EmbLayerNormPluginDynamic* EmbLayerNormPluginDynamic::deserialize(const std::str
     set_error(FWDMI_ERR_TRUNCATED, "EmbLayerNorm: serialized header truncated");
     return nullptr;
   }
-  if (!float_type((DataType)type) || ld <= 0 || t.word_count <= 0 || t.pos_count <= 0 || t.tok_count <= 0) {
+  // ld is bounded as in the LayerNorm plugin, so that the size below cannot wrap 64 bits
+  // (3 x 2^31 rows x 2^24 x 4 bytes < 2^59)
+  if (!float_type((DataType)type) || ld <= 0 || ld > (1 << 24) || t.word_count <= 0 || t.pos_count <= 0 ||
+      t.tok_count <= 0) {
     set_error(FWDMI_ERR_BAD_ARG, "EmbLayerNorm: serialized header malformed");
     return nullptr;
   }
@@ -490,6 +493,10 @@ EmbLayerNormPluginDynamic* EmbLayerNormPluginDynamic::deserialize(const std::str
   t.tok = read_table(t.tok_count);
   int32_t batch_major = 0;
   if (r.left() >= sizeof(int32_t)) r.pod(&batch_major);
+  if (!r.ok()) {
+    set_error(FWDMI_ERR_TRUNCATED, "EmbLayerNorm: serialized tables truncated");
+    return nullptr;
+  }
   return new EmbLayerNormPluginDynamic(name, (DataType)type, (DataType)mha, ld, std::move(t), eps, batch_major != 0);
 }
 

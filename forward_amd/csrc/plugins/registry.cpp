@@ -64,7 +64,8 @@ std::shared_ptr<HostDeviceBlob> HostDeviceBlob::map_file(const std::string& path
     return nullptr;
   }
   struct stat st {};
-  if (fstat(fd, &st) != 0 || (uint64_t)st.st_size < offset + nbytes) {
+  // compared without forming offset + nbytes, which a corrupt header could make wrap
+  if (fstat(fd, &st) != 0 || offset > (uint64_t)st.st_size || nbytes > (uint64_t)st.st_size - offset) {
     close(fd);
     set_error(FWDMI_ERR_TRUNCATED, "table file '%s' is shorter than offset %llu + %zu bytes", path.c_str(),
               (unsigned long long)offset, nbytes);

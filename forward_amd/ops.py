@@ -82,7 +82,9 @@ def embedding_bag(table, indices, offsets, mode="sum", per_sample_weights=None, 
         dst = out
     else:
         _dev(out, "out")
-        _require(out.dtype == odt and out.shape[0] == n_bags, 'out.dtype == odt and out.shape[0] == n_bags')
+        _require(out.dim() == 2 and out.dtype == odt and out.shape[0] == n_bags,
+                 'out is [n_bags, W] of the output dtype')
+        _require(0 <= out_col and out_col + dim <= out.shape[1], '0 <= out_col and out_col + dim <= out.shape[1]')
         stride = out.shape[1]
         dst = out.reshape(-1)[out_col:]
     psw = None
@@ -161,6 +163,7 @@ class MultiTableBatch:
             _require(self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype,
                      'self.indices[t].dtype == self.indices[0].dtype == self.offsets[t].dtype')
             _require(self.offsets[t].numel() == self.n_bags, 'self.offsets[t].numel() == self.n_bags')
+            _require(self.tables[t].dim() == 2 and self.tables[t].shape[0] > 0, 'every table is [rows > 0, dim]')
             _require((self.dim * self.tables[t].element_size()) % 16 != 0 or self.tables[t].data_ptr() % 16 == 0,
                      'tables of 16-byte-sliceable rows start on a 16-byte boundary')
             w = self.weights[t]
@@ -227,6 +230,7 @@ def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offse
                      'per_sample_weights[t] has the table dtype and one entry per id')
             desc[t, 7] = w.data_ptr()
         _require(tab.dim() == 2 and tab.shape[1] == dim and tab.dtype == tdt, 'tables share dim and dtype')
+        _require(tab.shape[0] > 0, 'every table is [rows > 0, dim]')
         _require((dim * tab.element_size()) % 16 != 0 or tab.data_ptr() % 16 == 0,
                  'tables of 16-byte-sliceable rows start on a 16-byte boundary')
         _require(ids.dim() == 1 and ids.dtype == idt and off.dtype == idt, 'ids are 1-D; ids and offsets share a dtype')
@@ -261,25 +265,36 @@ def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offse
     return out
 
 
-def _params(gamma, beta, bias=None):
+def _params(gamma, beta, bias=None, ld=None):
+    """gamma / beta (/ bias): fp32 device vectors of ``ld`` elements (the launchers index them by ld)."""
     g, b = _dev(gamma, "gamma"), _dev(beta, "beta")
     _require(g.dtype == torch.float32 and b.dtype == torch.float32,
              'g.dtype == torch.float32 and b.dtype == torch.float32')
     if bias is not None:
         _require(_dev(bias, "bias").dtype == torch.float32, '_dev(bias, "bias").dtype == torch.float32')
+    if ld is not None:
+        _require(g.numel() == ld and b.numel() == ld, 'gamma.numel() == beta.numel() == ld')
+        _require(bias is None or bias.numel() == ld, 'bias.numel() == ld')
     return g, b, bias
+
+
+def _out_like(out, ref, name="out"):
+    """A caller-supplied result buffer: device, contiguous, same dtype and element count as ``ref``."""
+    out = _dev(out, name)
+    _require(out.dtype == ref.dtype and out.numel() == ref.numel(),
+             '%s has the dtype and element count of the result' % name)
+    return out
 
 
 def skip_layer_norm(x, gamma, beta, skip=None, bias=None, eps=0.0, out=None, stream=None):
     """``LN(x (+ skip) (+ bias))`` over the last axis; gamma/beta/bias are fp32 device vectors."""
     x = _dev(x, "input")
-    g, b, bias = _params(gamma, beta, bias)
     ld = x.shape[-1]
-    _require(g.numel() == ld and b.numel() == ld, 'g.numel() == ld and b.numel() == ld')
+    g, b, bias = _params(gamma, beta, bias, ld)
     if skip is not None:
         _require(_dev(skip, "skip").shape == x.shape and skip.dtype == x.dtype,
                  '_dev(skip, "skip").shape == x.shape and skip.dtype == x.dtype')
-    out = torch.empty_like(x) if out is None else _dev(out, "out")
+    out = torch.empty_like(x) if out is None else _out_like(out, x)
     lib.check(lib.dll.fwdmi_skip_layer_norm(_stream(stream), ld, x.numel(), _p(x), _p(skip), _p(b), _p(g), _p(out),
                                             _p(bias), _FDT[x.dtype], eps))
     return out
@@ -287,9 +302,9 @@ def skip_layer_norm(x, gamma, beta, skip=None, bias=None, eps=0.0, out=None, str
 
 def layer_norm(x, gamma, beta, bias=None, eps=0.0, out=None, stream=None):
     x = _dev(x, "input")
-    g, b, bias = _params(gamma, beta, bias)
     ld = x.shape[-1]
-    out = torch.empty_like(x) if out is None else _dev(out, "out")
+    g, b, bias = _params(gamma, beta, bias, ld)
+    out = torch.empty_like(x) if out is None else _out_like(out, x)
     lib.check(lib.dll.fwdmi_layer_norm(_stream(stream), ld, x.numel(), _p(x), _p(b), _p(g), _p(out), _p(bias),
                                        _FDT[x.dtype], eps))
     return out
@@ -310,18 +325,29 @@ def emb_layer_norm(input_ids, segment_ids, input_mask, word, pos, tok, gamma, be
              'ids.dtype == torch.int32 and seg.dtype == torch.int32 and ids.dim() == 2 and seg.shape == ids.shape')
     word, pos, tok = _dev(word, "word"), _dev(pos, "pos"), _dev(tok, "tok")
     _require(word.dtype == pos.dtype == tok.dtype, 'word.dtype == pos.dtype == tok.dtype')
-    g, b, _ = _params(gamma, beta)
+    _require(word.dim() == 2 and pos.dim() == 2 and tok.dim() == 2 and pos.shape[1] == tok.shape[1] == word.shape[1],
+             'word, pos and tok are [rows, ld] with one ld')
     s, bsz = (ids.shape[1], ids.shape[0]) if batch_major else ids.shape
     ld = word.shape[1]
+    g, b, _ = _params(gamma, beta, None, ld)
+    _require(msk is None or (msk.dtype == torch.int32 and msk.shape == ids.shape),
+             'input_mask is int32 and shaped like input_ids')
     if out is None:
         out = torch.empty(tuple(ids.shape) + (ld,), dtype=word.dtype, device=word.device)
+    else:
+        out = _dev(out, "out")
+        _require(out.dtype == word.dtype and out.numel() == ids.numel() * ld, 'out holds ids.numel() * ld elements of the table dtype')
     if mask_idx is None and msk is not None:
         mask_idx = torch.empty((bsz,), dtype=torch.int32, device=word.device)
+    elif mask_idx is not None:
+        mask_idx = _dev(mask_idx, "mask_idx")
+        _require(mask_idx.dtype == torch.int32 and mask_idx.numel() == bsz, 'mask_idx is int32 [B]')
+        _require(msk is not None, 'mask_idx needs input_mask')
     x = lib.EmbExt()
     x.batch_major = 1 if batch_major else 0
     keep = []
     if skip is not None:
-        g2, b2, bias2 = _params(gamma2, beta2, bias2)
+        g2, b2, bias2 = _params(gamma2, beta2, bias2, ld)
         _require(_dev(skip, "skip").dtype == word.dtype and skip.numel() == ids.numel() * ld,
                  '_dev(skip, "skip").dtype == word.dtype and skip.numel() == ids.numel() * ld')
         if emb_out is not None:

@@ -141,7 +141,10 @@ int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t of
  * One table of a multi-table batch.  The array of these lives in DEVICE memory.
  */
 typedef struct fwdmi_bag_table {
-  const void* data;    /* [count, dim], 16-byte aligned when dim * element size is a multiple of 16 */
+  const void* data;    /* [count, dim], 16-byte aligned when dim * element size is a multiple of 16;
+                          must address count * dim elements.  count <= 0 is an empty table: data
+                          is not read (may be NULL), every id counts as out of range and the
+                          table's output block is zeros */
   const void* input;   /* [input_size] ids */
   const void* input_2; /* [n_bags] offsets (+1 with include_last_offset) */
   int64_t count;

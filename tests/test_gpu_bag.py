@@ -98,6 +98,51 @@ def test_config2_full_size_sum_fp16(oracle):
     assert_bits_equal(got, want, "config 2 fp16")
 
 
+@pytest.fixture(scope="module")
+def config2_full():
+    """Config 2 at its real size, generated once: 1 000 000 x 128 fp32 table, 4096 bags, Zipf ids,
+    per-sample weights.  The fp16 table is the rounded fp32 draw and the int64 ids are the int32
+    ones widened, exactly as workloads.config2 makes them, so every variant shares this draw."""
+    wl = workloads.config2(variant=0, table_dtype=np.float32, index_dtype=np.int32, weighted=True)
+    assert wl.table.shape == (1_000_000, 128) and wl.n_bags == 4096 and (wl.lengths == 0).sum() > 10
+    cache = {}
+
+    def tables(tdt):
+        if tdt not in cache:
+            host_t = wl.table.astype(tdt)
+            cache[tdt] = (host_t, dev(host_t))
+        return cache[tdt]
+    return wl, tables
+
+
+@pytest.mark.parametrize("tdt", [np.float32, np.float16])
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+@pytest.mark.parametrize("mode", ["sum", "mean", "max", "wsum"])
+def test_config2_full_size_every_variant(oracle, config2_full, tdt, idt, mode):
+    """Every table type x id type x mode of config 2 on the 1 M-row table, bit for bit against the
+    oracle (values, argmax ids, empty bags)."""
+    wl, tables = config2_full
+    host_t, dev_t = tables(tdt)
+    weighted = mode == "wsum"
+    m = "sum" if weighted else mode
+    idx, off = wl.indices.astype(idt), wl.offsets.astype(idt)
+    psw = wl.per_sample_weights.astype(tdt) if weighted else None
+    res = ops.embedding_bag(dev_t, dev(idx), dev(off), m, per_sample_weights=dev(psw), want_max_indices=(m == "max"))
+    want, warg, oob = oracle.embedding_bag(host_t, idx, off, OPS[m], per_sample_weights=psw,
+                                           want_max_indices=(m == "max"))
+    assert oob == 0
+    got = host(res[0] if m == "max" else res)
+    assert got.dtype == tdt and got.shape == (4096, 128)
+    assert_close(got, want, tdt, scale=0.05)
+    assert_bits_equal(got, want, "config 2 %s %s %s" % (np.dtype(tdt).name, np.dtype(idt).name, mode))
+    assert not got[wl.lengths == 0].any()
+    if m == "max":
+        arg = host(res[1])
+        assert arg.dtype == idt
+        np.testing.assert_array_equal(arg, warg)
+        assert_bits_equal(host(ops.embedding_bag(dev_t, dev(idx), dev(off), m)), want, "max, values only")
+
+
 @pytest.mark.parametrize("dim,tdt", [(1, np.float32), (2, np.float32), (4, np.float32), (10, np.float16),
                                      (64, np.float32), (100, np.float16), (200, np.float32), (1024, np.float16),
                                      (1100, np.float32), (2048, np.float32)])

@@ -180,3 +180,50 @@ def test_group_with_per_sample_weights(oracle, tdt):
         assert_bits_equal(out[:, t * dim:(t + 1) * dim], want, "launcher, table %d" % t)
     with pytest.raises(lib.FwdmiError, match="SUM"):
         batch.forward(mode="max")
+
+
+@pytest.mark.parametrize("count", [0, -3])
+@pytest.mark.parametrize("op", ["sum", "max"])
+def test_descriptor_of_a_table_without_rows(oracle, count, op):
+    """A descriptor with count <= 0 (and a null data pointer) handed straight to the C ABI: no row
+    address may be formed; the table's block is zeros, its ids count as out of range (flag set),
+    and the other tables of the launch are unaffected."""
+    import ctypes as C
+    from forward_amd import ops
+    rng = np.random.Generator(np.random.PCG64(77 + count))
+    rows, dim, n_bags = [300, 0, 4000], 128, 900
+    tables = [(rng.standard_normal((max(r, 1), dim)) * 0.3).astype(np.float16) for r in rows]
+    ids, offs = random_batch(rng, [300, 50, 4000], n_bags, np.int32)
+    d_tab = [dev(t) for t in tables]
+    d_ids, d_off = [dev(i) for i in ids], [dev(o) for o in offs]
+    desc = np.zeros((3, 8), np.int64)
+    for t in range(3):
+        desc[t] = (d_tab[t].data_ptr(), d_ids[t].data_ptr(), d_off[t].data_ptr(), rows[t], ids[t].size, 0, t * dim, 0)
+    desc[1, 0], desc[1, 3] = 0, count
+    d_desc = torch.from_numpy(desc).cuda()
+    for affinity in (0, lib.BAG_XCD_TABLE_AFFINITY):
+        out = torch.full((n_bags, 3 * dim), 7.0, dtype=torch.float16, device="cuda")
+        flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+        x = ops._ext(d_tab[0], d_ids[0], torch.float16, out_row_stride=3 * dim, oob_flag=flag, flags=affinity)
+        lib.check(lib.dll.fwdmi_embedding_bag_multi(C.c_void_p(d_desc.data_ptr()), 3, n_bags, C.c_void_p(out.data_ptr()),
+                                                    dim, ops.MODES[op], float(sum(i.size for i in ids)) / (3 * n_bags),
+                                                    C.byref(x), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        got = host(out)
+        assert int(flag.item()) == 1
+        assert not got[:, dim:2 * dim].any()
+        for t in (0, 2):
+            want, _, _ = oracle.embedding_bag(tables[t], ids[t], offs[t], ops.MODES[op])
+            assert_bits_equal(got[:, t * dim:(t + 1) * dim], want, "table %d beside the empty one" % t)
+    # bags of the empty table that hold no ids raise no flag
+    d_ids[1] = dev(np.zeros(1, np.int32))
+    desc[1, 1], desc[1, 2], desc[1, 4] = d_ids[1].data_ptr(), dev(np.zeros(n_bags, np.int32)).data_ptr(), 0
+    zero_off = dev(np.zeros(n_bags, np.int32))
+    desc[1, 2] = zero_off.data_ptr()
+    d_desc = torch.from_numpy(desc).cuda()
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = torch.full((n_bags, 3 * dim), 7.0, dtype=torch.float16, device="cuda")
+    x = ops._ext(d_tab[0], d_ids[0], torch.float16, out_row_stride=3 * dim, oob_flag=flag)
+    lib.check(lib.dll.fwdmi_embedding_bag_multi(C.c_void_p(d_desc.data_ptr()), 3, n_bags, C.c_void_p(out.data_ptr()), dim,
+                                                ops.MODES[op], 4.0, C.byref(x),
+                                                C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    assert int(flag.item()) == 0 and not host(out)[:, dim:2 * dim].any()

@@ -86,6 +86,10 @@ def test_table_by_file_reference_host_side(tmp_path):
     # a file that is too short, a missing file, both 'data' and 'data_file'
     with pytest.raises(lib.FwdmiError, match="shorter"):
         c.createPlugin("emb", fields[:6] + [F("data_file_row_offset", 50)])
+    # a corrupt file offset in the blob (offset + size would wrap 64 bits) is "too short", not a mapping
+    for off in (2**64 - 8, 2**64 - 1, 2**63):
+        with pytest.raises(lib.FwdmiError, match="shorter"):
+            c.deserializePlugin("emb", blob[:-8] + struct.pack("<Q", off))
     os.remove(tf)
     with pytest.raises(lib.FwdmiError, match="cannot open"):
         c.deserializePlugin("emb", blob)

@@ -303,6 +303,14 @@ def test_emb_layer_norm_plugin_host_contract():
     assert c.deserializePlugin("e", blob).serialize() == blob and p.clone().serialize() == blob
     with pytest.raises(lib.FwdmiError):
         c.deserializePlugin("e", blob[:-1])
+    # crafted headers: sizes whose product would wrap 64 bits, or that the blob cannot hold, are
+    # refused with a status (never an allocation failure inside a noexcept call)
+    for ld, word, pos, tok in ((2**31 - 1, 2**31 - 1, 2**31 - 1, 2**31 - 1), (2**24 + 1, 40, 12, 2),
+                               (16, 2**31 - 1, 12, 2), (2**24, 2**31 - 1, 2**31 - 1, 2**31 - 1), (0, 40, 12, 2),
+                               (16, -1, 12, 2)):
+        bad = struct.pack("<6if", lib.F16, lib.F16, ld, word, pos, tok, 0.0) + blob[28:]
+        with pytest.raises(lib.FwdmiError):
+            c.deserializePlugin("e", bad)
     # batch-major variant: [B,S] ids, [B,S,H,1,1] output, one trailing int in the blob
     bm = c.createPlugin("embeddings", fields + [F("batch_major", 1)])
     assert bm.getOutputDimensions(0, [(4, 12)] * 3) == [4, 12, 16, 1, 1] and bm.getOutputDimensions(1, [(4, 12)] * 3) == [4, 1]

@@ -28,6 +28,7 @@
 #include <algorithm>
 #include <climits>
 #include <cmath>
+#include <mutex>
 #include <type_traits>
 
 #include "../common.h"
@@ -641,6 +642,35 @@ __global__ __launch_bounds__(64) void bag_tables_fill_kernel(const TableChunk c,
   if (i < n) dst[i] = c.t[i];
 }
 
+// ---- scratch of the entry point that allocates nothing ---------------------------------------
+// The multi-table kernel reads its table descriptors from device memory.  Callers that cannot
+// allocate (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc) get
+// that memory from this array, which the loaded code object carries: every GPU the library runs
+// on holds its own copy, at its own address, until the process ends.
+constexpr int kNoAllocMaxTables = 1024;  // 64 KiB of descriptors
+static __device__ __align__(256) unsigned char scratch[kNoAllocMaxTables * sizeof(fwdmi_bag_table)];
+
+// In host code `scratch` is only a handle for the runtime, not a device address: the address on
+// the current device comes from hipGetSymbolAddress, once per device, and is kept here.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_on_current_device(fwdmi_bag_table** out) {
+  int dev = -1;
+  FWDMI_HIP_CHECK(hipGetDevice(&dev));
+  FWDMI_REQUIRE(dev >= 0 && dev < kMaxDevices, "no-allocation entry point: device index %d beyond %d", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    FWDMI_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    FWDMI_REQUIRE(p != nullptr, "no-allocation entry point: the scratch array has no address on device %d", dev);
+    g_scratch_ptr[dev] = p;
+  }
+  *out = static_cast<fwdmi_bag_table*>(g_scratch_ptr[dev]);
+  return FWDMI_OK;
+}
+
 struct BagShape {
   int grid, block;
   size_t lds;
@@ -920,6 +950,49 @@ int fwdmi_bag_tables_fill(const fwdmi_bag_table* tables_host, int32_t n_tables, 
     FWDMI_HIP_CHECK(hipGetLastError());
   }
   return FWDMI_OK;
+}
+
+int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_t n_tables, int64_t n_bags,
+                                      void* output, int32_t dim, int32_t op_type, double avg_bag_len,
+                                      const fwdmi_bag_ext* ext, void* stream) {
+  fwdmi::clear_error();
+  if (!tables_host || n_tables <= 0)
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "multi-table bags (no allocation): null or empty table array");
+  if (n_tables > fwdmi::kNoAllocMaxTables)
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG,
+                            "multi-table bags (no allocation): %d tables exceed the built-in descriptor "
+                            "buffer of %d; use fwdmi_embedding_bag_multi with a descriptor array of your own",
+                            n_tables, fwdmi::kNoAllocMaxTables);
+  if (ext && ext->per_sample_weights)
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG,
+                            "multi-table bags: per-sample weights go into the table descriptors "
+                            "(FWDMI_BAG_TABLE_WEIGHTS), not into ext->per_sample_weights");
+  // the descriptors are host memory here, so what the device form leaves to its caller is checked
+  const size_t sw = ext ? fwdmi::dtype_size(ext->table_dtype) : sizeof(float);
+  const size_t so = ext ? fwdmi::dtype_size(ext->out_dtype) : sizeof(float);
+  const int64_t stride = ext && ext->out_row_stride > 0 ? ext->out_row_stride : dim;
+  for (int32_t t = 0; t < n_tables; ++t) {
+    const fwdmi_bag_table& d = tables_host[t];
+    FWDMI_REQUIRE(d.count <= 0 || d.data, "multi-table bags (no allocation): table %d has rows but no data", t);
+    FWDMI_REQUIRE(d.input_size >= 0 && (d.input_size == 0 || d.input) && d.input_2,
+                  "multi-table bags (no allocation): table %d lacks ids or offsets", t);
+    FWDMI_REQUIRE(d.out_col >= 0 && dim > 0 && d.out_col + dim <= stride,
+                  "multi-table bags (no allocation): table %d writes columns %lld.. beyond the row of %lld", t,
+                  (long long)d.out_col, (long long)stride);
+    if (sw && ((size_t)dim * sw) % 16 == 0) {  // rows are read (and written) as 16-byte slices
+      const size_t store_align = std::min<size_t>(16, 16 / sw * so);
+      FWDMI_REQUIRE(reinterpret_cast<uintptr_t>(d.data) % 16 == 0 && ((size_t)d.out_col * so) % store_align == 0,
+                    "multi-table bags (no allocation): table %d: data or output column not aligned to its slices", t);
+    }
+  }
+  fwdmi_bag_table* dev_tables = nullptr;
+  if (const int rc = fwdmi::scratch_on_current_device(&dev_tables)) return rc;
+  // stream order keeps a call's descriptors intact until its launch has read them, as long as
+  // every call on this GPU uses the same stream (or the caller orders them)
+  if (const int rc = fwdmi_bag_tables_fill(tables_host, n_tables, dev_tables, stream)) return rc;
+  fwdmi_bag_table none{};
+  return fwdmi::bag_dispatch(dev_tables, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, ext,
+                             static_cast<hipStream_t>(stream));
 }
 
 // Measured on the 26-table configuration (tables of 0.25 MB .. 2.5 GB): per-bag cost ratios

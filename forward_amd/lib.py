@@ -88,6 +88,8 @@ SIGNATURES = {
     "fwdmi_bag_table_cost": (C.c_int, [_vp, _i32, _vp]),
     "fwdmi_bag_tables_fill": (C.c_int, [_vp, _i32, _vp, _vp]),
     "fwdmi_embedding_bag_multi": (C.c_int, [_vp, _i32, _i64, _vp, _i32, _i32, C.c_double, C.POINTER(BagExt), _vp]),
+    "fwdmi_embedding_bag_multi_noalloc": (C.c_int, [_vp, _i32, _i64, _vp, _i32, _i32, C.c_double, C.POINTER(BagExt),
+                                                    _vp]),
     "fwdmi_layer_norm": (C.c_int, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _i32, C.c_float]),
     "fwdmi_skip_layer_norm": (C.c_int, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i32, C.c_float]),
     "fwdmi_emb_layer_norm": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32,

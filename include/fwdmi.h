@@ -172,6 +172,23 @@ int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_table
                               const fwdmi_bag_ext* ext, void* stream);
 
 /*
+ * fwdmi_embedding_bag_multi for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  The descriptors are given in HOST memory; the library copies them (as kernel
+ * arguments, on `stream`) into a descriptor buffer that is part of its own code object, then
+ * launches exactly what fwdmi_embedding_bag_multi launches, so results are bit-identical.
+ * It calls no hipMalloc / hipFree or any other allocating routine; inputs and outputs are the
+ * caller's.  Limits: at most 1024 tables per call (more is FWDMI_ERR_BAD_ARG; the buffer holds
+ * 64 KiB per GPU for the life of the process).  Every call on one GPU shares that GPU's buffer:
+ * calls on the same stream are ordered by it; calls that overlap on one GPU (different streams
+ * without an ordering between them) race and must not be made.  The first call on a device looks
+ * the buffer's address up (hipGetSymbolAddress); make that call outside a graph capture.
+ */
+int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_t n_tables, int64_t n_bags,
+                                      void* output, int32_t dim, int32_t op_type, double avg_bag_len,
+                                      const fwdmi_bag_ext* ext, void* stream);
+
+/*
  * Writes n_tables descriptors from HOST memory into the DEVICE array a later
  * fwdmi_embedding_bag_multi on the same stream reads.  The descriptors travel as kernel
  * arguments: stream-ordered, no host synchronisation, no pinned staging buffer, and the host

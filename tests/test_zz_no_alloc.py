@@ -1,0 +1,101 @@
+"""fwdmi_embedding_bag_multi_noalloc: the multi-table launch for callers that cannot allocate
+device memory (its descriptor buffer is part of the library's code object).  Called through the
+C ABI and compared bit for bit with fwdmi_embedding_bag_multi on the same inputs, on two calls in
+a row, the second with a smaller input (fewer tables, fewer bags), so that what the first call
+left in the shared buffer must not leak into the second."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from forward_amd import lib, ops
+from gpu_util import assert_bits_equal, dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+def make_batch(rng, rows, n_bags, dim, tdt, idt, max_len):
+    tables = [(rng.standard_normal((r, dim)) * 0.3).astype(tdt) for r in rows]
+    ids, offs = [], []
+    for r in rows:
+        lengths = rng.integers(0, max_len, n_bags)
+        offs.append(np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(idt))
+        ids.append(rng.integers(0, r, int(lengths.sum())).astype(idt))
+    return tables, ids, offs
+
+
+def descriptors(d_tab, d_ids, d_off, dim):
+    desc = np.zeros((len(d_tab), 8), np.int64)
+    for t in range(len(d_tab)):
+        desc[t] = (d_tab[t].data_ptr(), d_ids[t].data_ptr(), d_off[t].data_ptr(), d_tab[t].shape[0],
+                   d_ids[t].numel(), 0, t * dim, 0)
+    return desc
+
+
+def launch_both(tables, ids, offs, dim, op, flags):
+    """(existing entry point's output, new entry point's output), each into its own buffer."""
+    d_tab, d_ids, d_off = [dev(t) for t in tables], [dev(i) for i in ids], [dev(o) for o in offs]
+    n_tables, n_bags = len(tables), offs[0].size
+    desc = descriptors(d_tab, d_ids, d_off, dim)
+    d_desc = torch.from_numpy(desc).cuda()
+    avg = float(sum(i.size for i in ids)) / max(1, n_tables * n_bags)
+    s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    outs = []
+    for entry, tab_arg in ((lib.dll.fwdmi_embedding_bag_multi, C.c_void_p(d_desc.data_ptr())),
+                           (lib.dll.fwdmi_embedding_bag_multi_noalloc, C.c_void_p(desc.ctypes.data))):
+        out = torch.full((n_bags, n_tables * dim), -3.0, dtype=d_tab[0].dtype, device="cuda")
+        x = ops._ext(d_tab[0], d_ids[0], d_tab[0].dtype, out_row_stride=n_tables * dim, flags=flags)
+        lib.check(entry(tab_arg, n_tables, n_bags, C.c_void_p(out.data_ptr()), dim, op, avg, C.byref(x), s))
+        outs.append(out)
+    torch.cuda.synchronize()
+    return host(outs[0]), host(outs[1])
+
+
+@pytest.mark.parametrize("tdt,idt", [(np.float16, np.int32), (np.float32, np.int64)])
+def test_no_alloc_entry_point_equals_the_allocating_form_twice_in_a_row(oracle, tdt, idt):
+    rng = np.random.Generator(np.random.PCG64(2024))
+    dim = 128 if tdt == np.float16 else 64
+    first = make_batch(rng, [4000, 17, 90000, 512, 30000, 7, 1200, 65000, 300], 3000, dim, tdt, idt, 24)
+    second = make_batch(rng, [900, 20000, 5], 257, dim, tdt, idt, 9)        # smaller: 3 tables, 257 bags
+    for call, (tables, ids, offs) in enumerate((first, second)):
+        for op in (ops.MODES["sum"], ops.MODES["max"]):
+            want, got = launch_both(tables, ids, offs, dim, op, lib.BAG_XCD_TABLE_AFFINITY if call == 0 else 0)
+            assert_bits_equal(got, want, "call %d op %d: no-allocation form against fwdmi_embedding_bag_multi" % (call, op))
+            for t, tab in enumerate(tables):                                  # and both against the oracle
+                ref, _, _ = oracle.embedding_bag(tab, ids[t], offs[t], op)
+                assert_bits_equal(got[:, t * dim:(t + 1) * dim], ref, "call %d table %d against the oracle" % (call, t))
+
+
+def test_no_alloc_entry_point_limits_and_argument_errors():
+    dim, n_bags = 32, 10
+    table, ids, off = dev(np.ones((8, dim), np.float32)), dev(np.zeros(10, np.int32)), dev(np.arange(10, dtype=np.int32))
+    out = torch.zeros((n_bags, dim), dtype=torch.float32, device="cuda")
+    s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    one = descriptors([table], [ids], [off], dim)
+    call = lambda desc, n, stride=0: lib.dll.fwdmi_embedding_bag_multi_noalloc(
+        C.c_void_p(desc.ctypes.data) if desc is not None else None, n, n_bags, C.c_void_p(out.data_ptr()), dim, 0, 1.0,
+        C.byref(ops._ext(table, ids, torch.float32, out_row_stride=stride)), s)
+    many = np.repeat(one, 1025, axis=0)
+    assert call(many, 1025) == lib.ERR_BAD_ARG and "1024" in lib.last_error()
+    assert call(None, 1) == lib.ERR_BAD_ARG
+    assert call(one, 0) == lib.ERR_BAD_ARG
+    bad = one.copy()
+    bad[0, 6] = 8                                                            # column block leaves the output row
+    assert call(bad, 1) == lib.ERR_BAD_ARG and "columns" in lib.last_error()
+    bad = one.copy()
+    bad[0, 0] = 0                                                            # rows but no data
+    assert call(bad, 1) == lib.ERR_BAD_ARG
+    assert call(one, 1) == lib.OK
+    torch.cuda.synchronize()
+    assert host(out).tolist() == [[1.0] * dim] * n_bags                      # ids are all 0, bags of one id
+    # the limit itself works: 1024 descriptors of the same small table, column blocks side by side
+    wide = torch.zeros((n_bags, 1024 * dim), dtype=torch.float32, device="cuda")
+    full = np.repeat(one, 1024, axis=0)
+    full[:, 6] = np.arange(1024) * dim
+    rc = lib.dll.fwdmi_embedding_bag_multi_noalloc(C.c_void_p(full.ctypes.data), 1024, n_bags, C.c_void_p(wide.data_ptr()),
+                                                   dim, 0, 1.0, C.byref(ops._ext(table, ids, torch.float32,
+                                                                                  out_row_stride=1024 * dim)), s)
+    assert rc == lib.OK, lib.last_error()
+    torch.cuda.synchronize()
+    assert bool((wide == 1.0).all())

@@ -47,5 +47,29 @@ __device__ __forceinline__ void gstore(T FWDMI_GLOBAL* p, const Pack<T, N>& r) {
     *(V FWDMI_GLOBAL*)p = x;
   }
 }
+// The same store (8, 16 or 32 bytes) with the non-temporal hint: the line is streamed through L2 instead of
+// staying there as a dirty line that displaces table rows.  For results far larger than the L2s.
+// Written as the instruction itself: a builtin store next to a plain store of the same value (one
+// per branch of a run-time choice) is merged with it by the optimiser and loses the hint.
+template <typename T, int N>
+__device__ __forceinline__ void gstore_stream(T FWDMI_GLOBAL* p, const Pack<T, N>& r) {
+  constexpr int kBytes = (int)sizeof(Pack<T, N>);
+  static_assert(kBytes == 8 || kBytes == 16 || kBytes == 32, "packs of 8, 16 or 32 bytes");
+  typedef uint32_t U4 __attribute__((ext_vector_type(4)));
+  typedef uint32_t U2 __attribute__((ext_vector_type(2)));
+  if constexpr (kBytes == 8) {
+    U2 x;
+    __builtin_memcpy(&x, &r, 8);
+    asm volatile("global_store_dwordx2 %0, %1, off nt" ::"v"(p), "v"(x) : "memory");
+  } else {
+    U4 x;
+    __builtin_memcpy(&x, &r, 16);
+    asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(p), "v"(x) : "memory");
+    if constexpr (kBytes == 32) {
+      __builtin_memcpy(&x, reinterpret_cast<const char*>(&r) + 16, 16);
+      asm volatile("global_store_dwordx4 %0, %1, off offset:16 nt" ::"v"(p), "v"(x) : "memory");
+    }
+  }
+}
 
 }  // namespace fwdmi

@@ -63,6 +63,15 @@ def parse():
                     help="bags per table in the CPU baseline sample (default: the whole batch)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device-to-device copy (known traffic, to scale rocprof byte counters)")
+    ap.add_argument("--replay", action="store_true",
+                    help="instead of the benchmark: the workload's row-id stream replayed as a plain gather (no "
+                         "bags), without and with result stores, beside the product launch (a table on stdout)")
+    ap.add_argument("--ids", default="zipf", choices=["zipf", "equal", "uniform"],
+                    help="--replay only: keep the workload's ids, or replace them (lengths kept) by one row per "
+                         "table / by uniform random rows")
+    ap.add_argument("--lru-sim", action="store_true",
+                    help="no GPU: rows fetched by an LRU cache of one XCD's L2 size over each table's id stream "
+                         "(the floor of the re-fetch ratio for table-at-a-time processing)")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the benchmark: single-table bag reduction over row widths, table types and "
                          "bag lengths with uniform random ids beside torch's GPU embedding_bag, then SkipLayerNorm "
@@ -509,8 +518,112 @@ def sweep_layer_norm(torch, ops):
                     rows, ld, "f16" if tdt == torch.float16 else "f32", ms, nbytes / ms / 1e6, tms, tms / ms), flush=True)
 
 
+def replay(torch, ops, workloads, lib, ids_mode):
+    """The workload's id stream as a plain gather (forward_amd/csrc/microbench/replay_gather.hip):
+    what the memory system charges for the rows alone, for the rows plus as many stored bytes as
+    the product writes, and for stores that never leave L2; beside the product launch on the same
+    ids.  Times are medians of HIP-event durations over 60 launches."""
+    import ctypes as C
+    path = os.path.join(ROOT, "forward_amd", "libfwdmi_microbench.so")
+    if not os.path.exists(path):
+        raise SystemExit("build the measurement aid first: make -C forward_amd/csrc microbench")
+    dll = C.CDLL(path)
+    wl = workloads.config4()
+    rng = np.random.Generator(np.random.PCG64(1))
+    for t in range(len(wl.rows)):
+        n = wl.indices[t].size
+        if ids_mode == "equal":
+            wl.indices[t] = np.zeros(n, np.int32)
+        elif ids_mode == "uniform":
+            wl.indices[t] = rng.integers(0, wl.rows[t], n).astype(np.int32)
+    tabs = device_tables(wl, torch)
+    idx = [torch.from_numpy(i).cuda() for i in wl.indices]
+    off = [torch.from_numpy(o).cuda() for o in wl.offsets]
+    batch = ops.MultiTableBatch(tabs, idx, off)
+    out = torch.zeros((wl.n_bags, batch.width), dtype=torch.float16, device="cuda")
+    for _ in range(300):
+        batch.forward(out=out, xcd_table_affinity=True)
+    _, per = time_events(torch, lambda: batch.forward(out=out, xcd_table_affinity=True), 60, 10)
+    print("ids: %s" % ids_mode)
+    print("%-72s %8.4f ms" % ("product launch (bags, ordered by length, %d result rows of 256 B)" %
+                              (wl.n_bags * len(wl.rows)), float(np.median(per))), flush=True)
+    del out, batch
+    chunk = 2600                      # ids per workgroup, as the product's runs of 160 bags x 16.3 ids
+    it_t, it_s, it_c = [], [], []
+    for t in range(len(wl.rows)):
+        n = wl.indices[t].size
+        for s0 in range(0, n, chunk):
+            it_t.append(t), it_s.append(s0), it_c.append(min(chunk, n - s0))
+    n_items = len(it_t)
+    cost = ops.MultiTableBatch(tabs, idx, off).default_table_cost()
+    c = np.cumsum(cost[np.array(it_t)] * np.array(it_c))
+    c /= c[-1]
+    xs = [0] + [int(np.searchsorted(c, k / 8.0)) for k in range(1, 8)] + [n_items]
+    longest = max(xs[k + 1] - xs[k] for k in range(8))
+
+    class Args(C.Structure):
+        _fields_ = [("tables", C.c_void_p), ("item_table", C.c_void_p), ("item_start", C.c_void_p),
+                    ("item_count", C.c_void_p), ("out", C.c_void_p), ("xcd_start", C.c_int32 * 9),
+                    ("store_every", C.c_int32), ("store_mode", C.c_int32), ("one", C.c_float)]
+    td = np.zeros((len(tabs), 2), np.int64)
+    for t in range(len(tabs)):
+        td[t] = (tabs[t].data_ptr(), idx[t].data_ptr())
+    d_td = torch.from_numpy(td).cuda()
+    d_t, d_s, d_c = (torch.tensor(a, dtype=torch.int32).cuda() for a in (it_t, it_s, it_c))
+    buf = torch.zeros((n_items * 16 * 64, 128), dtype=torch.float16, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    avg_len = wl.n_indices() / float(wl.n_bags * len(wl.rows))
+    every = int(round(avg_len / 8.0)) * 8          # whole 8-row steps: 16 rows per result for config 4
+    for label, store_every, mode in (
+            ("gather only (one result row per slot)", 0, 1),
+            ("gather + a 256 B result row every %d rows, plain stores" % every, every, 1),
+            ("gather + a 256 B result row every %d rows, non-temporal stores" % every, every, 2),
+            ("gather + a 256 B result row every %d rows, stores confined to 4 MiB (never leave L2)" % every, every, 3)):
+        a = Args(d_td.data_ptr(), d_t.data_ptr(), d_s.data_ptr(), d_c.data_ptr(), buf.data_ptr(),
+                 (C.c_int32 * 9)(*xs), store_every, mode, 1.0)
+
+        def fn():
+            rc = dll.fwdmi_mb_replay_gather(C.byref(a), longest, stream)
+            if rc:
+                raise RuntimeError("replay launch failed: hipError %d" % rc)
+        _, per = time_events(torch, fn, 60, 10)
+        print("%-72s %8.4f ms" % (label, float(np.median(per))), flush=True)
+
+
+def lru_sim(workloads, capacities=(8192, 12288, 16384, 32768)):
+    """Rows an LRU cache of `capacity` 256-byte rows fetches over each table's id stream in bag
+    order (one table at a time, as an XCD works through it): a 4 MiB L2 holds 16384 rows if it held
+    nothing else."""
+    from collections import OrderedDict
+    wl = workloads.config4()
+    distinct = sum(int(np.unique(i).size) for i in wl.indices)
+    print("ids %d, distinct rows %d" % (wl.n_indices(), distinct), flush=True)
+    for cap in capacities:
+        t0, miss = time.time(), 0
+        for ids in wl.indices:
+            cache = OrderedDict()
+            for r in ids.tolist():
+                if r in cache:
+                    cache.move_to_end(r)
+                else:
+                    miss += 1
+                    cache[r] = None
+                    if len(cache) > cap:
+                        cache.popitem(last=False)
+        print("capacity %6d rows (%4.1f MiB): %8d rows fetched = %.2f x the distinct rows  (%.0f s)" %
+              (cap, cap * 256 / 2**20, miss, miss / distinct, time.time() - t0), flush=True)
+
+
 def main():
     args = parse()
+    if args.record_traffic:
+        record_traffic(*args.record_traffic)
+        return
+    if args.lru_sim:
+        sys.path.insert(0, ROOT)
+        from forward_amd import workloads as _wl   # imports torch (CPU is enough) through the package
+        lru_sim(_wl)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (got --gpus %d)" % args.gpus,
               file=sys.stderr)
@@ -523,6 +636,10 @@ def main():
     if args.sweep:
         sweep(torch, ops)
         sweep_layer_norm(torch, ops)
+        return
+    if args.replay:
+        from forward_amd import lib
+        replay(torch, ops, workloads, lib, args.ids)
         return
 
     t0 = time.time()

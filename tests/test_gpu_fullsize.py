@@ -45,6 +45,41 @@ def test_sampled_bags_match_oracle_bit_exact(full, oracle):
         assert_bits_equal(got, want, "table %d (%d rows)" % (t, wl.rows[t]))
 
 
+@pytest.mark.parametrize("mode", ["mean", "max", "wsum"])
+def test_other_modes_sampled_bags_match_oracle_bit_exact(full, oracle, mode):
+    """The fused launch in its other modes at full size (mean, max, per-sample weights through the
+    table descriptors; int64 ids for max): sampled bags of every table against the oracle."""
+    wl, tabs, idx, off, batch, _ = full
+    weighted = mode == "wsum"
+    m = "sum" if weighted else mode
+    psw = None
+    if weighted:
+        g = torch.Generator(device="cuda").manual_seed(4004)
+        psw = [torch.rand(i.numel(), generator=g, device="cuda").half() for i in idx]
+        b = ops.MultiTableBatch(tabs, idx, off, per_sample_weights=psw)
+    elif mode == "max":
+        b = ops.MultiTableBatch(tabs, [i.long() for i in idx], [o.long() for o in off])
+    else:
+        b = batch
+    out = b.forward(mode=m, xcd_table_affinity=True)
+    torch.cuda.synchronize()
+    rng = np.random.Generator(np.random.PCG64(45))
+    for t in range(26):
+        ends = np.append(wl.offsets[t][1:], wl.indices[t].size).astype(np.int64)
+        lens = ends - wl.offsets[t]
+        bags = np.unique(np.concatenate([rng.integers(0, 65536, 200), np.argsort(lens)[-10:], [0, 65535]]))
+        pos = np.concatenate([np.arange(wl.offsets[t][x], ends[x]) for x in bags])
+        ids = wl.indices[t][pos]
+        uniq, inv = np.unique(ids, return_inverse=True)
+        rows = host(tabs[t][torch.from_numpy(uniq.astype(np.int64)).cuda()])
+        sub_off = workloads.offsets_from_lengths(lens[bags], np.int32)
+        w = host(psw[t][torch.from_numpy(pos).cuda()]) if weighted else None
+        want, _, oob = oracle.embedding_bag(rows, inv.astype(np.int32), sub_off, ops.MODES[m], per_sample_weights=w)
+        assert oob == 0
+        got = host(out[torch.from_numpy(bags).cuda(), t * 128:(t + 1) * 128])
+        assert_bits_equal(got, want, "%s, table %d (%d rows)" % (mode, t, wl.rows[t]))
+
+
 def test_fused_equals_per_table_and_int64(full):
     wl, tabs, idx, off, batch, out = full
     ref = torch.zeros_like(out)

@@ -99,3 +99,25 @@ def test_no_alloc_entry_point_limits_and_argument_errors():
     assert rc == lib.OK, lib.last_error()
     torch.cuda.synchronize()
     assert bool((wide == 1.0).all())
+
+
+def test_no_alloc_entry_point_on_config4_at_full_size():
+    """The whole 26-table configuration (65536 bags per table, 8 GB of tables) through the
+    no-allocation entry point equals the fused launch of fwdmi_embedding_bag_multi bit for bit."""
+    from forward_amd import workloads
+    wl = workloads.config4()
+    tabs = [wl.device_table(t, torch) for t in range(26)]
+    idx = [torch.from_numpy(i).cuda() for i in wl.indices]
+    off = [torch.from_numpy(o).cuda() for o in wl.offsets]
+    batch = ops.MultiTableBatch(tabs, idx, off)
+    want = batch.forward(xcd_table_affinity=True)
+    desc = batch.desc.cpu().numpy()
+    got = torch.zeros_like(want)
+    x = ops._ext(tabs[0], idx[0], torch.float16, out_row_stride=want.shape[1], flags=lib.BAG_XCD_TABLE_AFFINITY,
+                 table_cost=batch.default_table_cost())
+    lib.check(lib.dll.fwdmi_embedding_bag_multi_noalloc(C.c_void_p(desc.ctypes.data), 26, wl.n_bags,
+                                                        C.c_void_p(got.data_ptr()), 128, 0,
+                                                        wl.n_indices() / (26.0 * wl.n_bags), C.byref(x),
+                                                        C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)

@@ -48,6 +48,9 @@ constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting 
 #ifndef FWDMI_BAG_UNROLL
 #define FWDMI_BAG_UNROLL 8
 #endif
+#ifndef FWDMI_BAG_STREAM_BYTES
+#define FWDMI_BAG_STREAM_BYTES (8.0 * 1048576.0)  // results of at least this size are stored with the non-temporal hint
+#endif
 #ifndef FWDMI_BAG_WAVES_PER_EU
 #define FWDMI_BAG_WAVES_PER_EU 6  // register budget of 80 VGPRs: measured best on the 26-table configuration
 #endif
@@ -835,10 +838,12 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                 ((out_stride * so) % store_align) == 0 &&
                 (tables_dev || (single.out_col * so) % store_align == 0);
 
-  // A result much larger than the eight 4 MiB L2s cannot be found there by whoever reads it next; written
-  // with the non-temporal hint it does not displace table rows on its way out either (measured on the
-  // 26-table configuration: 2.8 % off the launch, 19 % when every row hits in cache).
-  if (L.vec_store && (double)n_bags * n_tables * dim * so >= 64.0 * 1048576.0) L.vec_store = 2;
+  // A result of several MiB does not survive in the 4 MiB L2 of the XCD that wrote it until somebody
+  // reads it (and a reader on another XCD would not find it there anyway); written with the
+  // non-temporal hint it does not displace table rows on its way out.  Measured: 2.8 % off the
+  // 26-table launch (19 % when every row hits in cache), 3.8 % off 26 single-table launches of
+  // 16 MiB results each; a reader of a 16 MiB result right behind the launch costs 2 % more.
+  if (L.vec_store && (double)n_bags * n_tables * dim * so >= FWDMI_BAG_STREAM_BYTES) L.vec_store = 2;
 
   const bool weighted = x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS));
   FWDMI_REQUIRE(!x.square_sum_out || (op == FWDMI_OP_SUM && !weighted),

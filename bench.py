@@ -336,7 +336,12 @@ def plugin_level(torch, wl, tabs, idx, off, want):
     from forward_amd import lib, plugin
     from forward_amd.plugin import PluginFieldData as F
     res = {}
+    need = sum(t.numel() * t.element_size() for t in tabs)
     shm = "/dev/shm" if os.path.isdir("/dev/shm") and os.access("/dev/shm", os.W_OK) else None
+    if shm is not None:
+        st = os.statvfs(shm)
+        if st.f_bavail * st.f_frsize < need + (1 << 30):
+            shm = None                     # too small for the tables: the default temporary directory then
     fd, path = tempfile.mkstemp(prefix="fwdmi_tables_", suffix=".bin", dir=shm)
     plugins = []
     try:

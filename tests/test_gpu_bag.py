@@ -505,3 +505,33 @@ def test_sum_and_square_sum_in_one_pass(oracle, tdt, idt):
     assert torch.equal(s, s2) and torch.equal(q, q2)
     with pytest.raises(lib.FwdmiError, match="with_square_sum"):
         c2.createPlugin("fm", bag_fields(table, op=3) + [F("with_square_sum", 1)])
+
+
+@pytest.mark.parametrize("tdt", [np.float32, np.float16])
+@pytest.mark.parametrize("odt", [np.float32, np.float16])
+def test_results_large_enough_for_streaming_stores(oracle, tdt, odt):
+    """Results of 8 MiB and more are written with non-temporal stores of 8, 16 or 32 bytes per
+    lane (table type x result type); plain bags, a column block of a wider matrix, max mode and the
+    two-output form all take that path here and must equal the oracle bit for bit."""
+    rng = np.random.Generator(np.random.PCG64(88))
+    rows, dim, n_bags = 3000, 128, 70000
+    table = (rng.standard_normal((rows, dim)) * 0.5).astype(tdt)
+    lengths = rng.integers(0, 4, n_bags)
+    idx = rng.integers(0, rows, int(lengths.sum())).astype(np.int32)
+    off = workloads.offsets_from_lengths(lengths, np.int32)
+    tod = torch.float16 if odt == np.float16 else torch.float32
+    assert n_bags * dim * np.dtype(odt).itemsize >= 8 << 20
+    for mode in ("sum", "max"):
+        want, _, _ = oracle.embedding_bag(table, idx, off, OPS[mode], out_dtype=odt)
+        got = host(ops.embedding_bag(dev(table), dev(idx), dev(off), mode, out_dtype=tod))
+        assert_bits_equal(got, want, "%s" % mode)
+    wide = torch.full((n_bags, 3 * dim), 5.0, dtype=tod, device="cuda")
+    ops.embedding_bag(dev(table), dev(idx), dev(off), "sum", out_dtype=tod, out=wide, out_col=dim)
+    w = host(wide)
+    want, _, _ = oracle.embedding_bag(table, idx, off, OPS["sum"], out_dtype=odt)
+    assert_bits_equal(w[:, dim:2 * dim], want, "column block")
+    assert (w[:, :dim] == 5.0).all() and (w[:, 2 * dim:] == 5.0).all()
+    s1, s2 = ops.embedding_bag(dev(table), dev(idx), dev(off), "sum", out_dtype=tod, with_square_sum=True)
+    want2, _, _ = oracle.embedding_bag(table, idx, off, OPS["square_sum"], out_dtype=odt)
+    assert_bits_equal(host(s1), want, "sum of the two-output form")
+    assert_bits_equal(host(s2), want2, "square sum of the two-output form")

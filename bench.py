@@ -523,36 +523,16 @@ def sweep_layer_norm(torch, ops):
                     rows, ld, "f16" if tdt == torch.float16 else "f32", ms, nbytes / ms / 1e6, tms, tms / ms), flush=True)
 
 
-def replay(torch, ops, workloads, lib, ids_mode):
-    """The workload's id stream as a plain gather (forward_amd/csrc/microbench/replay_gather.hip):
-    what the memory system charges for the rows alone, for the rows plus as many stored bytes as
-    the product writes, and for stores that never leave L2; beside the product launch on the same
-    ids.  Times are medians of HIP-event durations over 60 launches."""
+def replay_times(torch, ops, wl, tabs, idx, off, steps=60):
+    """Times (ms, median of HIP-event durations) of forward_amd/csrc/microbench/replay_gather.hip on the
+    workload's id stream: the rows alone, the rows plus as many stored bytes as the product writes
+    (plain / non-temporal stores), and with the stores confined to 4 MiB.  None when the measurement
+    aid is not built."""
     import ctypes as C
     path = os.path.join(ROOT, "forward_amd", "libfwdmi_microbench.so")
     if not os.path.exists(path):
-        raise SystemExit("build the measurement aid first: make -C forward_amd/csrc microbench")
+        return None
     dll = C.CDLL(path)
-    wl = workloads.config4()
-    rng = np.random.Generator(np.random.PCG64(1))
-    for t in range(len(wl.rows)):
-        n = wl.indices[t].size
-        if ids_mode == "equal":
-            wl.indices[t] = np.zeros(n, np.int32)
-        elif ids_mode == "uniform":
-            wl.indices[t] = rng.integers(0, wl.rows[t], n).astype(np.int32)
-    tabs = device_tables(wl, torch)
-    idx = [torch.from_numpy(i).cuda() for i in wl.indices]
-    off = [torch.from_numpy(o).cuda() for o in wl.offsets]
-    batch = ops.MultiTableBatch(tabs, idx, off)
-    out = torch.zeros((wl.n_bags, batch.width), dtype=torch.float16, device="cuda")
-    for _ in range(300):
-        batch.forward(out=out, xcd_table_affinity=True)
-    _, per = time_events(torch, lambda: batch.forward(out=out, xcd_table_affinity=True), 60, 10)
-    print("ids: %s" % ids_mode)
-    print("%-72s %8.4f ms" % ("product launch (bags, ordered by length, %d result rows of 256 B)" %
-                              (wl.n_bags * len(wl.rows)), float(np.median(per))), flush=True)
-    del out, batch
     chunk = 2600                      # ids per workgroup, as the product's runs of 160 bags x 16.3 ids
     it_t, it_s, it_c = [], [], []
     for t in range(len(wl.rows)):
@@ -578,12 +558,10 @@ def replay(torch, ops, workloads, lib, ids_mode):
     buf = torch.zeros((n_items * 16 * 64, 128), dtype=torch.float16, device="cuda")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     avg_len = wl.n_indices() / float(wl.n_bags * len(wl.rows))
-    every = int(round(avg_len / 8.0)) * 8          # whole 8-row steps: 16 rows per result for config 4
-    for label, store_every, mode in (
-            ("gather only (one result row per slot)", 0, 1),
-            ("gather + a 256 B result row every %d rows, plain stores" % every, every, 1),
-            ("gather + a 256 B result row every %d rows, non-temporal stores" % every, every, 2),
-            ("gather + a 256 B result row every %d rows, stores confined to 4 MiB (never leave L2)" % every, every, 3)):
+    every = max(8, int(round(avg_len / 8.0)) * 8)   # whole 8-row steps: 16 rows per result for config 4
+    res = {"rows_per_result_row": every}
+    for key, store_every, mode in (("gather_only_ms", 0, 1), ("gather_plain_stores_ms", every, 1),
+                                   ("gather_streaming_stores_ms", every, 2), ("gather_stores_within_4MiB_ms", every, 3)):
         a = Args(d_td.data_ptr(), d_t.data_ptr(), d_s.data_ptr(), d_c.data_ptr(), buf.data_ptr(),
                  (C.c_int32 * 9)(*xs), store_every, mode, 1.0)
 
@@ -591,8 +569,43 @@ def replay(torch, ops, workloads, lib, ids_mode):
             rc = dll.fwdmi_mb_replay_gather(C.byref(a), longest, stream)
             if rc:
                 raise RuntimeError("replay launch failed: hipError %d" % rc)
-        _, per = time_events(torch, fn, 60, 10)
-        print("%-72s %8.4f ms" % (label, float(np.median(per))), flush=True)
+        _, per = time_events(torch, fn, steps, 10)
+        res[key] = float(np.median(per))
+    return res
+
+
+def replay(torch, ops, workloads, ids_mode):
+    """`--replay`: the product launch beside the bag-free replay of the same id stream (a table on stdout)."""
+    wl = workloads.config4()
+    rng = np.random.Generator(np.random.PCG64(1))
+    for t in range(len(wl.rows)):
+        n = wl.indices[t].size
+        if ids_mode == "equal":
+            wl.indices[t] = np.zeros(n, np.int32)
+        elif ids_mode == "uniform":
+            wl.indices[t] = rng.integers(0, wl.rows[t], n).astype(np.int32)
+    tabs = device_tables(wl, torch)
+    idx = [torch.from_numpy(i).cuda() for i in wl.indices]
+    off = [torch.from_numpy(o).cuda() for o in wl.offsets]
+    batch = ops.MultiTableBatch(tabs, idx, off)
+    out = torch.zeros((wl.n_bags, batch.width), dtype=torch.float16, device="cuda")
+    for _ in range(300):
+        batch.forward(out=out, xcd_table_affinity=True)
+    _, per = time_events(torch, lambda: batch.forward(out=out, xcd_table_affinity=True), 60, 10)
+    print("ids: %s" % ids_mode)
+    print("%-72s %8.4f ms" % ("product launch (bags, ordered by length, %d result rows of 256 B)" %
+                              (wl.n_bags * len(wl.rows)), float(np.median(per))), flush=True)
+    del out, batch
+    r = replay_times(torch, ops, wl, tabs, idx, off)
+    if r is None:
+        raise SystemExit("build the measurement aid first: make -C forward_amd/csrc microbench")
+    e = r["rows_per_result_row"]
+    for label, key in (("gather only (one result row per slot)", "gather_only_ms"),
+                       ("gather + a 256 B result row every %d rows, plain stores" % e, "gather_plain_stores_ms"),
+                       ("gather + a 256 B result row every %d rows, non-temporal stores" % e, "gather_streaming_stores_ms"),
+                       ("gather + a 256 B result row every %d rows, stores confined to 4 MiB (never leave L2)" % e,
+                        "gather_stores_within_4MiB_ms")):
+        print("%-72s %8.4f ms" % (label, r[key]), flush=True)
 
 
 def lru_sim(workloads, capacities=(8192, 12288, 16384, 32768)):
@@ -643,8 +656,7 @@ def main():
         sweep_layer_norm(torch, ops)
         return
     if args.replay:
-        from forward_amd import lib
-        replay(torch, ops, workloads, lib, args.ids)
+        replay(torch, ops, workloads, args.ids)
         return
 
     t0 = time.time()
@@ -774,6 +786,16 @@ def main():
             result["plugin_level"] = plugin_level(torch, wl, tabs, idx, off, out)
         except Exception as e:  # noqa: BLE001  (a side measurement must not lose the headline)
             result["plugin_level"] = {"error": repr(e)}
+    if not args.no_extra and full:
+        # the same id stream as a plain gather that knows no bags and stores as many bytes: what the
+        # memory system charges for this workload with this lane mapping, measured in this run
+        try:
+            rt = replay_times(torch, ops, wl, tabs, idx, off, steps=40)
+            if rt:
+                rt["kernel_over_replay_with_streaming_stores"] = (ev_ms / rt["gather_streaming_stores_ms"])
+                result["replay_without_bags"] = rt
+        except Exception as e:  # noqa: BLE001
+            result["replay_without_bags"] = {"error": repr(e)}
     if not args.no_extra:
         del tabs, batch
         result["extra"] = extra_measurements(torch, ops, workloads, max(10, args.steps), with_cpu=not args.no_cpu)

@@ -121,3 +121,58 @@ def test_no_alloc_entry_point_on_config4_at_full_size():
                                                         C.c_void_p(torch.cuda.current_stream().cuda_stream)))
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+
+
+def test_no_alloc_entry_point_under_graph_capture(oracle):
+    """The callers the entry point is for: recorded into a HIP graph (no allocation may happen
+    there) and replayed with new ids in the same buffers, with eager calls of the same entry point
+    between the replays (they share the built-in descriptor buffer, in stream order)."""
+    rng = np.random.Generator(np.random.PCG64(31))
+    rows, dim, n_bags, n_ids = [700, 12000, 33], 64, 500, 6000
+    tables = [(rng.standard_normal((r, dim)) * 0.3).astype(np.float16) for r in rows]
+    d_tab = [dev(t) for t in tables]
+
+    def batch(seed):
+        r = np.random.Generator(np.random.PCG64(seed))
+        ids, offs = [], []
+        for rws in rows:
+            cuts = np.sort(r.integers(0, n_ids + 1, n_bags - 1))
+            offs.append(np.concatenate([[0], cuts]).astype(np.int32))          # fixed id count per table
+            ids.append(r.integers(0, rws, n_ids).astype(np.int32))
+        return ids, offs
+
+    ids0, offs0 = batch(0)
+    d_ids, d_off = [dev(i) for i in ids0], [dev(o) for o in offs0]
+    desc = descriptors(d_tab, d_ids, d_off, dim)
+    out = torch.zeros((n_bags, 3 * dim), dtype=torch.float16, device="cuda")
+    x = ops._ext(d_tab[0], d_ids[0], torch.float16, out_row_stride=3 * dim)
+
+    def launch(dst):
+        s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        lib.check(lib.dll.fwdmi_embedding_bag_multi_noalloc(C.c_void_p(desc.ctypes.data), 3, n_bags,
+                                                            C.c_void_p(dst.data_ptr()), dim, 0, n_ids / float(n_bags),
+                                                            C.byref(x), s))
+
+    def want(ids, offs):
+        return np.concatenate([oracle.embedding_bag(tables[t], ids[t], offs[t], 0)[0] for t in range(3)], axis=1)
+
+    launch(out)                                     # eager first: the buffer's address is looked up here
+    torch.cuda.synchronize()
+    assert_bits_equal(host(out), want(ids0, offs0), "eager")
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launch(out)
+    torch.cuda.synchronize()
+    other = torch.zeros_like(out)
+    for seed in (1, 2, 3):
+        ids, offs = batch(seed)
+        for t in range(3):
+            d_ids[t].copy_(dev(ids[t]))
+            d_off[t].copy_(dev(offs[t]))
+        out.fill_(-1.0)
+        g.replay()
+        torch.cuda.synchronize()
+        assert_bits_equal(host(out), want(ids, offs), "replay %d" % seed)
+        launch(other)                               # an eager call between the replays
+        torch.cuda.synchronize()
+        assert_bits_equal(host(other), want(ids, offs), "eager between replays %d" % seed)

@@ -468,6 +468,11 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
             ex["config2_sum_%s_pytorch_rocm_gpu" % tname] = {"bags_per_s": wl.n_bags / (ms_t * 1e-3), "ms": ms_t}
         except Exception as e:  # noqa: BLE001
             ex["config2_sum_%s_pytorch_rocm_gpu" % tname] = {"error": repr(e)}
+    # these kernels move their algorithmic bytes once (rocprofv3 FETCH_SIZE / WRITE_SIZE agree, see
+    # profiles/): the algorithmic rate over the HBM peak is their roofline position
+    for v in ex.values():
+        if isinstance(v, dict) and "algorithmic_GBs" in v:
+            v["frac_of_hbm_peak"] = v["algorithmic_GBs"] / HBM_PEAK_GBS
     return ex
 
 

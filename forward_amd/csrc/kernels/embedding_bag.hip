@@ -28,6 +28,7 @@
 #include <algorithm>
 #include <climits>
 #include <cmath>
+#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 
@@ -50,6 +51,9 @@ constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting 
 #endif
 #ifndef FWDMI_BAG_STREAM_BYTES
 #define FWDMI_BAG_STREAM_BYTES (8.0 * 1048576.0)  // results of at least this size are stored with the non-temporal hint
+#endif
+#ifndef FWDMI_BAG_TAIL_RUNS
+#define FWDMI_BAG_TAIL_RUNS(resident) ((resident) / 4)  // measured best on the 26-table configuration (16 .. 384 tried)
 #endif
 #ifndef FWDMI_BAG_WAVES_PER_EU
 #define FWDMI_BAG_WAVES_PER_EU 6  // register budget of 80 VGPRs: measured best on the 26-table configuration
@@ -87,6 +91,7 @@ struct BagLaunch {
   int32_t xcd_affinity;      // != 0: XCD x works through work items [xcd_start[x], xcd_start[x+1])
   int32_t xcd_start[kXcds + 1];
   int32_t total_wgs;
+  int32_t tail_runs;  // XCD mapping only: the last `tail_runs` runs of every XCD's segment are issued as four workgroups each
   int32_t idx_cap;    // 32-bit words of the LDS id window: that many row numbers, or half as many 64-bit ids
 };
 
@@ -108,10 +113,24 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   // placement (workgroup b runs on XCD b % 8) so that one XCD works through whole tables: a
   // table's hot rows are then fetched into one L2 instead of all eight.
   int work = blockIdx.x;
+  int quarter = -1;  // 0..3: this workgroup reduces that quarter of run `work`; -1: the whole run
   if (L.xcd_affinity) {
+    // A workgroup lives for about an eighth of the launch, so after an XCD has started its last
+    // run its CUs empty out for that long.  The last runs of a segment are therefore cut in four:
+    // their workgroups live a quarter as long and the XCD drains that much faster.
     const int x = (int)(blockIdx.x % kXcds);
-    work = L.xcd_start[x] + (int)(blockIdx.x / kXcds);
-    if (work >= L.xcd_start[x + 1]) return;
+    const int j = (int)(blockIdx.x / kXcds);
+    const int len = L.xcd_start[x + 1] - L.xcd_start[x];
+    const int tail = min(len, L.tail_runs);
+    const int whole = len - tail;
+    if (j < whole) {
+      work = L.xcd_start[x] + j;
+    } else {
+      const int jj = j - whole;
+      if (jj >= 4 * tail) return;
+      work = L.xcd_start[x] + whole + (jj >> 2);
+      quarter = jj & 3;
+    }
   }
   const int t = work / L.wgs_per_table;
   const int wg = work - t * L.wgs_per_table;
@@ -135,8 +154,10 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const int gl = tid & (G - 1);
   const int slots = wg_lanes >> L.log2_g;
 
-  const int64_t bag0 = (int64_t)wg * L.bags_per_wg;
-  const int nb = (int)min((int64_t)L.bags_per_wg, L.n_bags - bag0);
+  const int quarter_bags = L.bags_per_wg >> 2;  // the host keeps bags_per_wg a multiple of 4 when it cuts runs
+  const int64_t bag0 = (int64_t)wg * L.bags_per_wg + (quarter > 0 ? quarter * quarter_bags : 0);
+  const int nb = (int)min((int64_t)(quarter < 0 ? L.bags_per_wg : quarter_bags), L.n_bags - bag0);
+  if (nb <= 0) return;  // a quarter beyond the table's last bag (uniform over the workgroup)
   const TI FWDMI_GLOBAL* __restrict__ ids = gconst<TI>(T.input);
   // per-sample weights: the launch's (single table) or the table's own; none = weight 1
   const TW FWDMI_GLOBAL* __restrict__ psw = gconst<TW>(L.tables ? T.weights : L.psw);
@@ -819,7 +840,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   const int64_t total_bags = n_bags * n_tables;
   const int64_t target_wgs = (int64_t)device_cus() * 4;
   int64_t want_bags = std::max<int64_t>(1, total_bags / target_wgs);
-  const int64_t fit_bags = std::max<int64_t>(1, (int64_t)(max_cap / 1.5 / avg_len));
+  const int64_t fit_bags = std::max<int64_t>(1, (int64_t)(max_cap / 2.0 / avg_len));
   want_bags = std::min<int64_t>(std::min(want_bags, fit_bags), kMaxBagsPerWG);
   int block = kWG;
   while (block > 64 && block / 2 >= lanes && (int64_t)(block / 2 / lanes) >= want_bags * L.n_slices) block /= 2;
@@ -887,8 +908,22 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
       L.xcd_start[k] = cut;
       longest = std::max(longest, cut - L.xcd_start[k - 1]);
     }
-    FWDMI_REQUIRE((int64_t)longest * kXcds < (int64_t)1 << 31, "embedding bag: grid too large");
-    grid = longest * kXcds;
+    // Runs cut in four at the end of every segment (see the kernel): as many as a quarter of what an XCD holds
+    // at once, and only in launches that fill the chip several times over.
+    const int resident = device_cus() / kXcds * 6;  // workgroups of 256 lanes an XCD holds at the 6-per-CU occupancy
+    L.tail_runs = 0;
+    if (block == kWG && L.bags_per_wg % 4 == 0 && L.bags_per_wg / 4 >= slots && longest >= 4 * resident)
+      L.tail_runs = FWDMI_BAG_TAIL_RUNS(resident);
+#ifdef FWDMI_EXP_ENV
+    if (const char* e = getenv("FWDMI_EXP_TAIL_RUNS")) L.tail_runs = atoi(e);
+#endif
+    int most = 0;  // workgroups of the XCD with the most
+    for (int k = 0; k < kXcds; ++k) {
+      const int len = L.xcd_start[k + 1] - L.xcd_start[k];
+      most = std::max(most, len + 3 * std::min(len, L.tail_runs));
+    }
+    FWDMI_REQUIRE((int64_t)most * kXcds < (int64_t)1 << 31, "embedding bag: grid too large");
+    grid = most * kXcds;
   }
   const bool f16 = x.table_dtype == FWDMI_F16, i64 = x.index_dtype == FWDMI_I64;
   const BagShape sh{grid, block, bag_lds_bytes(L, kind == kWeighted)};

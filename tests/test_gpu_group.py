@@ -227,3 +227,40 @@ def test_descriptor_of_a_table_without_rows(oracle, count, op):
                                                 ops.MODES[op], 4.0, C.byref(x),
                                                 C.c_void_p(torch.cuda.current_stream().cuda_stream)))
     assert int(flag.item()) == 0 and not host(out)[:, dim:2 * dim].any()
+
+
+@pytest.mark.parametrize("tdt,idt", [(np.float32, np.int32), (np.float16, np.int64)])
+def test_quarter_runs_at_segment_ends_on_ragged_tables(oracle, tdt, idt):
+    """A launch large enough for the XCD mapping to cut the last runs of every segment in four
+    (several hundred runs per XCD), on shapes that make those quarters ragged: a bag count that
+    leaves a table's last run with one bag (three of its quarters are empty), segment cuts in the
+    middle of tables (uneven costs) and at table ends (equal costs), a bag too long for the id
+    window inside a tail run, empty bags, ids outside the table.  Whole output against the oracle."""
+    from forward_amd import ops
+    rng = np.random.Generator(np.random.PCG64(1234))
+    n_tables, n_bags = 8, 80001
+    dim = 64 if tdt == np.float32 else 128          # 16 lanes per row either way: 16 bags in flight per workgroup
+    rows = [int(r) for r in rng.integers(5, 30000, n_tables)]
+    tables = [(rng.standard_normal((r, dim)) * 0.3).astype(tdt) for r in rows]
+    ids, offs = [], []
+    for t, r in enumerate(rows):
+        lengths = rng.integers(0, 60, n_bags)      # mean 29.5: runs of 64 bags, quarters of 16
+        lengths[-1] = 40
+        lengths[n_bags - 20] = 5000                 # inside the table's last runs: that quarter reads its ids unstaged
+        offs.append(np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(idt))
+        i = rng.integers(0, r, int(lengths.sum()))
+        i[rng.integers(0, i.size, 50)] = r + 3      # outside the table: skipped
+        ids.append(i.astype(idt))
+    d_tab, d_ids, d_off = [dev(t) for t in tables], [dev(i) for i in ids], [dev(o) for o in offs]
+    want = np.zeros((n_bags, n_tables * dim), tdt)
+    for t in range(n_tables):
+        oracle.embedding_bag(tables[t], ids[t], offs[t], oracle.OP_SUM, out=want, out_col=dim * t)
+    batch = ops.MultiTableBatch(d_tab, d_ids, d_off)
+    plain = host(batch.forward())
+    assert_bits_equal(plain, want, "without the XCD mapping")
+    for name, cost in (("equal costs", np.ones(n_tables)), ("uneven costs", 1.0 + 0.6 * rng.random(n_tables))):
+        flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+        got = batch.forward(out=torch.full((n_bags, n_tables * dim), 3.0, dtype=d_tab[0].dtype, device="cuda"),
+                            xcd_table_affinity=True, table_cost=cost, oob_flag=flag)
+        assert_bits_equal(host(got), want, name)
+        assert int(flag.item()) == 1

@@ -95,6 +95,30 @@ struct BagLaunch {
   int32_t idx_cap;    // 32-bit words of the LDS id window: that many row numbers, or half as many 64-bit ids
 };
 
+// Hands elements first[0 .. n) to put(i, value), the workgroup's lanes sharing the work.  Long
+// ranges come in with 16-byte loads (a load instruction occupies the CU's memory pipeline for the
+// same time whatever its width); the elements before the first 16-byte boundary and behind the
+// last one go one by one, so nothing outside the range is read.  `first` is aligned to its type.
+template <typename T, typename Put>
+__device__ __forceinline__ void stream_in(const T FWDMI_GLOBAL* first, int n, int tid, int lanes, Put put) {
+  constexpr int kPer = 16 / (int)sizeof(T);
+  if (n < 2 * lanes) {  // uniform over the workgroup: too short for the split to pay
+    for (int i = tid; i < n; i += lanes) put(i, first[i]);
+    return;
+  }
+  const int misalign = (int)((reinterpret_cast<uintptr_t>(first) & 15) / sizeof(T));
+  const int head = (kPer - misalign) & (kPer - 1);
+  const int n_vec = (n - head) / kPer;
+  const int body_end = head + n_vec * kPer;
+  for (int v = tid; v < n_vec; v += lanes) {
+    const Pack<T, kPer> p = gload<T, kPer>(first + head + v * kPer);
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) put(head + v * kPer + e, p.v[e]);
+  }
+  if (tid < head) put(tid, first[tid]);
+  if (body_end + tid < n) put(body_end + tid, first[body_end + tid]);
+}
+
 template <typename TW, typename TI, int VEC, int KIND>
 __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(const BagLaunch L) {
   // LDS carve-up (dynamic, sized by the host): offsets | ids | weights | lengths | order
@@ -220,15 +244,21 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const int window = compact ? L.idx_cap : L.idx_cap / (int)(sizeof(TI) / 4);
   const bool staged = span >= 0 && span <= window;  // uniform over the workgroup
   if (staged) {
-    for (int i = tid; i < span; i += wg_lanes) {
-      const TI id = ids[span0 + i];
+    auto put = [&](int i, TI id) {
       if (compact) {
         const uint64_t row = (uint64_t)((int64_t)id - T.data_offset);
         s_row[i] = row < (uint64_t)T.count ? (uint32_t)row : 0xFFFFFFFFu;
       } else {
         s_idx[i] = id;
       }
-      if (KIND == kWeighted) s_w[i] = has_w ? (float)psw[span0 + i] : 1.0f;
+    };
+    stream_in<TI>(ids + span0, (int)span, tid, wg_lanes, put);
+    if (KIND == kWeighted) {
+      if (has_w) {
+        stream_in<TW>(psw + span0, (int)span, tid, wg_lanes, [&](int i, TW w) { s_w[i] = (float)w; });
+      } else {
+        for (int i = tid; i < span; i += wg_lanes) s_w[i] = 1.0f;
+      }
     }
   }
   // ---- order the run's bags by length, longest first --------------------------------------

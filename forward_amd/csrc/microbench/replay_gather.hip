@@ -3,7 +3,7 @@
 // those rows in that order from what the bag structure (lengths, ordering, per-bag results) adds.
 //
 // Same shape as the product kernel where it matters for memory behaviour: a 256-lane workgroup
-// owns a contiguous chunk of one table's ids, copies them into LDS, and sixteen 16-lane slots read
+// owns a contiguous chunk of one table's ids, copies them into LDS (16-byte loads), and sixteen 16-lane slots read
 // 256-byte fp16 rows with 128-bit loads, eight in flight per lane, fp32 accumulation; workgroups
 // are dealt to the eight XCDs in contiguous segments of the table-major work list.  There are no
 // bags: a slot sums a contiguous part of the chunk and (optionally) stores a 256-byte result row
@@ -56,7 +56,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6))) void r
   const int32_t FWDMI_MB_GLOBAL* ids = (const int32_t FWDMI_MB_GLOBAL*)tp->ids;
   const char FWDMI_MB_GLOBAL* tab = (const char FWDMI_MB_GLOBAL*)tp->data;
   const int tid = threadIdx.x;
-  for (int i = tid; i < n; i += 256) s_row[i] = (uint32_t)ids[s0 + i];
+  {
+    // 16-byte loads like the product kernel's staging pass; the ends of the chunk go id by id
+    const int32_t FWDMI_MB_GLOBAL* first = ids + s0;
+    const int head = min(n, (int)((4 - ((reinterpret_cast<uintptr_t>(first) >> 2) & 3)) & 3));
+    const int n_vec = (n - head) / 4;
+    for (int v = tid; v < n_vec; v += 256) {
+      const U4 q = *(const U4 FWDMI_MB_GLOBAL*)(first + head + 4 * v);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s_row[head + 4 * v + e] = q[e];
+    }
+    if (tid < head) s_row[tid] = (uint32_t)first[tid];
+    const int done = head + 4 * n_vec;
+    if (done + tid < n) s_row[done + tid] = (uint32_t)first[done + tid];
+  }
   __syncthreads();
   const int slot = tid >> 4, gl = tid & 15;
   const int per = (n + 15) / 16;

@@ -535,3 +535,37 @@ def test_results_large_enough_for_streaming_stores(oracle, tdt, odt):
     want2, _, _ = oracle.embedding_bag(table, idx, off, OPS["square_sum"], out_dtype=odt)
     assert_bits_equal(host(s1), want, "sum of the two-output form")
     assert_bits_equal(host(s2), want2, "square sum of the two-output form")
+
+
+@pytest.mark.parametrize("tdt,idt", [(np.float16, np.int32), (np.float32, np.int64)])
+def test_ids_and_weights_at_every_alignment(oracle, tdt, idt):
+    """A run's ids and weights are staged with 16-byte loads between the first and the last 16-byte
+    boundary and one by one outside them: id and weight arrays that start 0 .. 3 (ids) and 0 .. 7
+    (fp16 weights) elements past a 16-byte boundary, runs long enough for the wide loads, bit-exact
+    for sum and for weighted sum.  The elements before and behind the arrays hold ids outside the
+    table and NaN weights: reading one would raise the flag or poison a bag."""
+    rng = np.random.Generator(np.random.PCG64(515))
+    rows, dim, n_bags = 5000, 64, 90000      # runs of some 80 bags, 1500 ids
+    table = (rng.standard_normal((rows, dim)) * 0.3).astype(tdt)
+    lengths = rng.integers(0, 40, n_bags)
+    n = int(lengths.sum())
+    off = np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(idt)
+    ids = rng.integers(0, rows, n).astype(idt)
+    psw = rng.random(n).astype(tdt)
+    want, _, _ = oracle.embedding_bag(table, ids, off, oracle.OP_SUM)
+    want_w, _, _ = oracle.embedding_bag(table, ids, off, oracle.OP_SUM, per_sample_weights=psw)
+    d_tab, d_off = dev(table), dev(off)
+    for shift in range(16 // ids.itemsize):
+        for wshift in sorted({0, 1, 16 // psw.itemsize - 1, shift}):
+            pad_i = np.full(n + 16, rows + 7, idt)
+            pad_i[shift:shift + n] = ids
+            pad_w = np.full(n + 16, np.nan, tdt)
+            pad_w[wshift:wshift + n] = psw
+            d_ids, d_w = dev(pad_i)[shift:shift + n], dev(pad_w)[wshift:wshift + n]
+            assert d_ids.data_ptr() % 16 == (shift * ids.itemsize) % 16
+            flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+            got = ops.embedding_bag(d_tab, d_ids, d_off, "sum", oob_flag=flag)
+            assert_bits_equal(host(got), want, "ids %d elements past a 16-byte boundary" % shift)
+            got = ops.embedding_bag(d_tab, d_ids, d_off, "sum", per_sample_weights=d_w, oob_flag=flag)
+            assert_bits_equal(host(got), want_w, "ids +%d, weights +%d elements" % (shift, wshift))
+            assert int(flag.item()) == 0

@@ -58,9 +58,10 @@ constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting 
 #ifndef FWDMI_BAG_WAVES_PER_EU
 #define FWDMI_BAG_WAVES_PER_EU 6  // register budget of 80 VGPRs: measured best on the 26-table configuration
 #endif
-// argmax tracking and weights carry more live registers: they keep the looser budget
+// argmax tracking and the second accumulator carry more live registers: they keep the looser budget;
+// the weighted form sits in between (measured on the 26-table configuration: 4 -> 5 wavefronts 2 % faster)
 #define FWDMI_BAG_OCCUPANCY \
-  __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kWeighted || KIND == kSumSq) ? 4 : FWDMI_BAG_WAVES_PER_EU)))
+  __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kSumSq) ? 4 : KIND == kWeighted ? 5 : FWDMI_BAG_WAVES_PER_EU)))
 constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 
 // kMax also tracks the argmax (needs max_indices); kMaxValue is the plugin's case: values only
@@ -880,6 +881,17 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   L.bags_per_wg = (int)std::max<int64_t>(1, std::min<int64_t>(kMaxBagsPerWG, units / L.n_slices));
   L.idx_cap = std::min(max_cap, std::max(64, next_pow2((int)std::min<double>(max_cap, avg_len * L.bags_per_wg * 2.0)))) *
               (wide_ids ? 2 : 1);
+  // With per-sample weights every window slot also holds a weight, and at twice the expected ids the
+  // two windows (35 KiB for a run of 112 bags) leave a CU four workgroups.  The expected ids plus 5.5
+  // times the spread of a sum of `bags_per_wg` lengths whose deviation equals their mean keeps all
+  // but one run in ten thousand staged (a run that reads its ids unstaged takes several times as
+  // long: at 4 spreads, 0.25 % of the runs unstaged, the launch below measures 0.466 ms); measured on
+  // the 26-table configuration: 0.490 -> 0.440 ms together with the register budget above.
+  if (x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS))) {
+    const double ids = avg_len * (L.bags_per_wg + 5.5 * std::sqrt((double)L.bags_per_wg));
+    const int tight = ((int)std::min<double>(max_cap, std::max(64.0, ids)) + 63) / 64 * 64 * (wide_ids ? 2 : 1);
+    L.idx_cap = std::min(L.idx_cap, tight);
+  }
   const int64_t wgs = (n_bags + L.bags_per_wg - 1) / L.bags_per_wg;
   FWDMI_REQUIRE(wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
   L.wgs_per_table = (int)wgs;

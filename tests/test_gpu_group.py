@@ -264,3 +264,37 @@ def test_quarter_runs_at_segment_ends_on_ragged_tables(oracle, tdt, idt):
                             xcd_table_affinity=True, table_cost=cost, oob_flag=flag)
         assert_bits_equal(host(got), want, name)
         assert int(flag.item()) == 1
+
+
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+def test_tables_of_very_different_bag_lengths(oracle, idt):
+    """One-hot tables beside tables of long bags in one launch: runs are sized from the mean bag
+    length of the whole launch, so a run of a long-bag table holds several times the ids the id
+    window takes and reads its ids unstaged.  With weights too; whole output against the oracle."""
+    from forward_amd import ops
+    rng = np.random.Generator(np.random.PCG64(77))
+    dim, n_bags = 64, 30000
+    rows = [9000, 400, 20000, 70, 3000, 1500]
+    mean_len = [1, 90, 1, 40, 1, 150]
+    tables = [(rng.standard_normal((r, dim)) * 0.3).astype(np.float16) for r in rows]
+    ids, offs, psw = [], [], []
+    for r, m in zip(rows, mean_len):
+        lengths = np.ones(n_bags, np.int64) if m == 1 else rng.poisson(m, n_bags)
+        if m == 150:
+            lengths[1000:1010] = 7000          # longer than the window by themselves
+            lengths[5::97] = 0
+        offs.append(np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(idt))
+        ids.append(rng.integers(0, r, int(lengths.sum())).astype(idt))
+        psw.append(rng.random(ids[-1].size).astype(np.float16))
+    d_tab, d_ids, d_off = [dev(t) for t in tables], [dev(i) for i in ids], [dev(o) for o in offs]
+    for weights in (None, psw):
+        want = np.zeros((n_bags, len(rows) * dim), np.float16)
+        for t in range(len(rows)):
+            oracle.embedding_bag(tables[t], ids[t], offs[t], oracle.OP_SUM, out=want, out_col=dim * t,
+                                 per_sample_weights=None if weights is None else weights[t])
+        batch = ops.MultiTableBatch(d_tab, d_ids, d_off,
+                                    per_sample_weights=None if weights is None else [dev(w) for w in weights])
+        for affinity in (False, True):
+            got = batch.forward(out=torch.full((n_bags, len(rows) * dim), 3.0, dtype=torch.float16, device="cuda"),
+                                xcd_table_affinity=affinity)
+            assert_bits_equal(host(got), want, "weights %s, affinity %s" % (weights is not None, affinity))

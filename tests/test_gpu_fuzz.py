@@ -167,3 +167,67 @@ def test_random_table_groups(oracle, seed):
         want, _, _ = oracle.embedding_bag(tables[t], ids[t], offs[t], ORACLE_OP[mode], per_sample_weights=psw[t],
                                           include_last_offset=include_last, out_dtype=odt)
         assert_bits_equal(got[:, t * dim:(t + 1) * dim], want, "seed %d table %d of %d (%s)" % (seed, t, n_tables, mode))
+
+
+def _offset_copy(a, k):
+    """``a`` on the device, starting ``k`` elements past an allocation boundary."""
+    if a is None:
+        return None
+    big = torch.empty(a.size + 8, dtype=torch.from_numpy(a[:0]).dtype, device="cuda")
+    big[k:k + a.size] = torch.from_numpy(a).cuda()
+    return big[k:k + a.size]
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_large_batches(oracle, seed):
+    """Batches of 2 500 ... 200 000 bags (runs of hundreds of bags: ids staged with wide loads, bags
+    ordered by length, the XCD mapping with its quarter runs where the launch is large enough), bag
+    lengths from four distributions including a heavy tail, id and weight arrays that start off a
+    16-byte boundary, one table or a group: every column block bit-identical to the oracle's."""
+    r = np.random.Generator(np.random.PCG64(424200 + seed))
+    n_tables = int(r.choice([1, 1, 2, 3, 8, 12]))
+    dim = int(r.choice([8, 32, 64, 128, 256]))
+    tdt = r.choice([np.float32, np.float16])
+    idt = r.choice([np.int32, np.int64])
+    n_bags = int(r.choice([5000, 30000, 70001, 200000])) // (2 if n_tables > 3 else 1)
+    mode = MODES[int(r.integers(0, 4))]
+    weighted = mode == "sum" and r.random() < 0.4
+    include_last = bool(r.random() < 0.3)
+    tables, ids, offs, psw = [], [], [], []
+    for t in range(n_tables):
+        rows = int(r.choice([3, 700, 90000]))
+        tables.append((r.standard_normal((rows, dim)) * 0.5).astype(tdt))
+        style = int(r.integers(0, 4))
+        if style == 0:
+            lengths = r.integers(0, 4, n_bags)
+        elif style == 1:
+            lengths = r.integers(0, 50, n_bags)
+        elif style == 2:
+            lengths = np.minimum((r.pareto(1.2, n_bags) + 1).astype(np.int64), 3000)
+        else:
+            lengths = r.poisson(int(r.choice([2, 20, 80])), n_bags)
+        lengths = lengths.astype(np.int64)
+        n = int(lengths.sum())
+        off = np.concatenate([[0], np.cumsum(lengths)])
+        offs.append((off if include_last else off[:-1]).astype(idt))
+        i = r.integers(0, rows, n)
+        if r.random() < 0.3 and n:
+            i[r.integers(0, n, 20)] = rows + 5
+        ids.append(i.astype(idt))
+        psw.append(r.random(n).astype(tdt) if weighted and r.random() < 0.8 else None)
+    odt = tdt if r.random() < 0.7 else (np.float16 if tdt == np.float32 else np.float32)
+    tt = torch.float16 if odt == np.float16 else torch.float32
+    shift = int(r.integers(0, 4))
+    d_ids = [_offset_copy(i, shift) for i in ids]
+    d_psw = [_offset_copy(w, (shift * 3) % 8) for w in psw] if weighted else None
+    if n_tables == 1:
+        got = host(ops.embedding_bag(dev(tables[0]), d_ids[0], dev(offs[0]), mode, include_last_offset=include_last,
+                                     out_dtype=tt, per_sample_weights=d_psw[0] if weighted else None))
+    else:
+        got = host(ops.embedding_bag_group([dev(t) for t in tables], d_ids, [dev(o) for o in offs], mode,
+                                           include_last_offset=include_last, out_dtype=tt,
+                                           xcd_table_affinity=bool(seed % 2), per_sample_weights=d_psw))
+    for t in range(n_tables):
+        want, _, _ = oracle.embedding_bag(tables[t], ids[t], offs[t], ORACLE_OP[mode], per_sample_weights=psw[t],
+                                          include_last_offset=include_last, out_dtype=odt)
+        assert_bits_equal(got[:, t * dim:(t + 1) * dim], want, "seed %d table %d of %d (%s)" % (seed, t, n_tables, mode))

@@ -46,6 +46,7 @@ constexpr int kWG = 256;           // lanes per workgroup (large batches; small 
 constexpr int kIdxBytes = FWDMI_BAG_IDX_BYTES;   // LDS bytes of the id window per workgroup (4096 row numbers / 2048 64-bit ids)
 constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
 constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting sort
+constexpr int kMaxVarTables = 64;  // tables of a launch whose runs may differ in size from table to table
 #ifndef FWDMI_BAG_UNROLL
 #define FWDMI_BAG_UNROLL 8
 #endif
@@ -94,6 +95,11 @@ struct BagLaunch {
   int32_t total_wgs;
   int32_t tail_runs;  // XCD mapping only: the last `tail_runs` runs of every XCD's segment are issued as four workgroups each
   int32_t idx_cap;    // 32-bit words of the LDS id window: that many row numbers, or half as many 64-bit ids
+  // Multi-table launches whose tables differ in mean bag length: table t's runs hold run_bags[t] bags and
+  // are work items [run_start[t], run_start[t + 1]); bags_per_wg is then the largest of them (it sizes LDS).
+  int32_t var_runs;
+  int32_t run_start[kMaxVarTables + 1];
+  uint16_t run_bags[kMaxVarTables];
 };
 
 // Hands elements first[0 .. n) to put(i, value), the workgroup's lanes sharing the work.  Long
@@ -157,8 +163,17 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
       quarter = jj & 3;
     }
   }
-  const int t = work / L.wgs_per_table;
-  const int wg = work - t * L.wgs_per_table;
+  int t, wg, bpw;  // table, run of the table, bags of a run of this table: uniform over the workgroup
+  if (L.var_runs) {
+    t = 0;
+    while (work >= L.run_start[t + 1]) ++t;  // at most kMaxVarTables steps over kernel arguments
+    wg = work - L.run_start[t];
+    bpw = L.run_bags[t];
+  } else {
+    t = work / L.wgs_per_table;
+    wg = work - t * L.wgs_per_table;
+    bpw = L.bags_per_wg;
+  }
   fwdmi_bag_table T;
   if (L.tables) {
     const fwdmi_bag_table FWDMI_GLOBAL* tp = gconst<fwdmi_bag_table>(L.tables) + t;
@@ -179,9 +194,9 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const int gl = tid & (G - 1);
   const int slots = wg_lanes >> L.log2_g;
 
-  const int quarter_bags = L.bags_per_wg >> 2;  // the host keeps bags_per_wg a multiple of 4 when it cuts runs
-  const int64_t bag0 = (int64_t)wg * L.bags_per_wg + (quarter > 0 ? quarter * quarter_bags : 0);
-  const int nb = (int)min((int64_t)(quarter < 0 ? L.bags_per_wg : quarter_bags), L.n_bags - bag0);
+  const int quarter_bags = bpw >> 2;  // the host keeps run sizes multiples of 4 when it cuts runs
+  const int64_t bag0 = (int64_t)wg * bpw + (quarter > 0 ? quarter * quarter_bags : 0);
+  const int nb = (int)min((int64_t)(quarter < 0 ? bpw : quarter_bags), L.n_bags - bag0);
   if (nb <= 0) return;  // a quarter beyond the table's last bag (uniform over the workgroup)
   const TI FWDMI_GLOBAL* __restrict__ ids = gconst<TI>(T.input);
   // per-sample weights: the launch's (single table) or the table's own; none = weight 1
@@ -876,25 +891,68 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   int block = kWG;
   while (block > 64 && block / 2 >= lanes && (int64_t)(block / 2 / lanes) >= want_bags * L.n_slices) block /= 2;
   const int slots = block / lanes;
-  // a whole number of rounds over the slots
-  int64_t units = std::max<int64_t>(slots, want_bags * L.n_slices / slots * slots);
-  L.bags_per_wg = (int)std::max<int64_t>(1, std::min<int64_t>(kMaxBagsPerWG, units / L.n_slices));
-  L.idx_cap = std::min(max_cap, std::max(64, next_pow2((int)std::min<double>(max_cap, avg_len * L.bags_per_wg * 2.0)))) *
-              (wide_ids ? 2 : 1);
-  // With per-sample weights every window slot also holds a weight, and at twice the expected ids the
-  // two windows (35 KiB for a run of 112 bags) leave a CU four workgroups.  The expected ids plus 5.5
-  // times the spread of a sum of `bags_per_wg` lengths whose deviation equals their mean keeps all
-  // but one run in ten thousand staged (a run that reads its ids unstaged takes several times as
-  // long: at 4 spreads, 0.25 % of the runs unstaged, the launch below measures 0.466 ms); measured on
-  // the 26-table configuration: 0.490 -> 0.440 ms together with the register budget above.
-  if (x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS))) {
-    const double ids = avg_len * (L.bags_per_wg + 5.5 * std::sqrt((double)L.bags_per_wg));
-    const int tight = ((int)std::min<double>(max_cap, std::max(64.0, ids)) + 63) / 64 * 64 * (wide_ids ? 2 : 1);
-    L.idx_cap = std::min(L.idx_cap, tight);
+  // Bags of a run and words of its id window for bags of `avg` ids on average.
+  const bool weighted_launch = x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS));
+  auto size_run = [&](double avg, int64_t want, int* bags, int* cap) {
+    // a whole number of rounds over the slots
+    const int64_t units = std::max<int64_t>(slots, want * L.n_slices / slots * slots);
+    *bags = (int)std::max<int64_t>(1, std::min<int64_t>(kMaxBagsPerWG, units / L.n_slices));
+    *cap = std::min(max_cap, std::max(64, next_pow2((int)std::min<double>(max_cap, avg * *bags * 2.0)))) * (wide_ids ? 2 : 1);
+    // With per-sample weights every window slot also holds a weight, and at twice the expected ids the
+    // two windows (35 KiB for a run of 112 bags) leave a CU four workgroups.  The expected ids plus 5.5
+    // times the spread of a sum of `bags` lengths whose deviation equals their mean keeps all
+    // but one run in ten thousand staged (a run that reads its ids unstaged takes several times as
+    // long: at 4 spreads, 0.25 % of the runs unstaged, the launch below measures 0.466 ms); measured on
+    // the 26-table configuration: 0.490 -> 0.440 ms together with the register budget above.
+    if (weighted_launch) {
+      const double ids = avg * (*bags + 5.5 * std::sqrt((double)*bags));
+      const int tight = ((int)std::min<double>(max_cap, std::max(64.0, ids)) + 63) / 64 * 64 * (wide_ids ? 2 : 1);
+      *cap = std::min(*cap, tight);
+    }
+  };
+  size_run(avg_len, want_bags, &L.bags_per_wg, &L.idx_cap);
+  // Tables whose mean bag lengths differ (one-hot features beside multi-hot ones) get runs of their
+  // own size: sized from the launch's mean, the runs of a long-bag table overflow the id window and
+  // those of a one-hot table hold a few ids each.  Measured on 13 one-hot + 13 long-bag tables
+  // (28.6 M ids): 0.562 ms with one run size.
+  int run_bags[kMaxVarTables];
+  bool var_runs = false;
+  if (tables_dev && x.table_avg_len && n_tables > 1 && n_tables <= kMaxVarTables) {
+    const int64_t want_all = std::min<int64_t>(std::max<int64_t>(1, total_bags / target_wgs), kMaxBagsPerWG);
+    int lo = INT_MAX, hi = 0, cap_max = 0;
+    for (int t = 0; t < n_tables; ++t) {
+      const double a = (double)x.table_avg_len[t];
+      FWDMI_REQUIRE(a >= 0.0 && a < 1e30, "embedding bag: table_avg_len must be finite and not negative");
+      const double avg_t = std::max(1.0, a);
+      const int64_t fit_t = std::max<int64_t>(1, (int64_t)(max_cap / 2.0 / avg_t));
+      int cap_t = 0;
+      size_run(avg_t, std::min(want_all, fit_t), &run_bags[t], &cap_t);
+      lo = std::min(lo, run_bags[t]);
+      hi = std::max(hi, run_bags[t]);
+      cap_max = std::max(cap_max, cap_t);
+    }
+    if (2 * hi >= 3 * lo) {  // otherwise one size serves all tables
+      var_runs = true;
+      L.bags_per_wg = hi;
+      L.idx_cap = cap_max;
+    }
   }
   const int64_t wgs = (n_bags + L.bags_per_wg - 1) / L.bags_per_wg;
   FWDMI_REQUIRE(wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
   L.wgs_per_table = (int)wgs;
+  int64_t total_runs = wgs * n_tables;
+  L.var_runs = 0;
+  if (var_runs) {
+    total_runs = 0;
+    for (int t = 0; t < n_tables; ++t) {
+      L.run_start[t] = (int32_t)total_runs;
+      L.run_bags[t] = (uint16_t)run_bags[t];
+      total_runs += (n_bags + run_bags[t] - 1) / run_bags[t];
+      FWDMI_REQUIRE(total_runs < (int64_t)1 << 31, "embedding bag: grid too large");
+    }
+    L.run_start[n_tables] = (int32_t)total_runs;
+    L.var_runs = 1;
+  }
   const size_t store_align = std::min<size_t>(16, VEC * so);
   L.vec_store = VEC > 1 && (reinterpret_cast<uintptr_t>(output) % store_align) == 0 &&
                 (reinterpret_cast<uintptr_t>(x.square_sum_out) % store_align) == 0 &&
@@ -908,7 +966,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   // 16 MiB results each; a reader of a 16 MiB result right behind the launch costs 2 % more.
   if (L.vec_store && (double)n_bags * n_tables * dim * so >= FWDMI_BAG_STREAM_BYTES) L.vec_store = 2;
 
-  const bool weighted = x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS));
+  const bool weighted = weighted_launch;
   FWDMI_REQUIRE(!x.square_sum_out || (op == FWDMI_OP_SUM && !weighted),
                 "embedding bag: square_sum_out needs op SUM without per-sample weights");
   const int kind = op == FWDMI_OP_MAX      ? (x.max_indices ? kMax : kMaxValue)
@@ -917,45 +975,82 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                    : x.square_sum_out          ? kSumSq
                                                : kPlain;
   L.psw = x.per_sample_weights;
-  int grid = (int)(wgs * n_tables);
+  int grid = (int)total_runs;
   L.total_wgs = grid;
   L.xcd_affinity = 0;
   if (tables_dev && n_tables > 1 && (x.flags & FWDMI_BAG_XCD_TABLE_AFFINITY)) {
     // Cut the table-major work list into eight contiguous segments of equal estimated cost
     // (equal length when the caller gives no per-table cost).
     L.xcd_affinity = 1;
+    // A bag costs its rows plus a constant (result store, bookkeeping) worth kBagRows rows: fixed-length
+    // launches of 1 .. 64 rows per bag fit rows / 36.6 TB/s + result bytes / 3.7 TB/s, and one-hot
+    // tables beside tables of 33 ids per bag measure 1 : 4.1 per bag.  With every table's mean bag
+    // length known the caller's per-bag cost is scaled by it; without, all tables count as equally long.
+    constexpr double kBagRows = 9.6;
+    auto cost_of = [&](int u) {
+      double c = x.table_cost ? (double)x.table_cost[u] : 1.0;
+      if (x.table_avg_len) c *= (std::max(0.0, (double)x.table_avg_len[u]) + kBagRows) / (avg_len + kBagRows);
+      return c;
+    };
     double total = 0.0;
     for (int t = 0; t < n_tables; ++t) {
-      const double c = x.table_cost ? (double)x.table_cost[t] : 1.0;
+      const double c = cost_of(t);
       FWDMI_REQUIRE(c > 0.0 && c < 1e30, "embedding bag: table_cost must be positive and finite");
-      total += c * (double)wgs;
+      const double a = x.table_avg_len ? (double)x.table_avg_len[t] : 0.0;
+      FWDMI_REQUIRE(a >= 0.0 && a < 1e30, "embedding bag: table_avg_len must be finite and not negative");
+      total += cost_of(t) * (double)wgs;
     }
     int t = 0;
     double before = 0.0;  // cost of the tables before t
     int longest = 0;
     L.xcd_start[0] = 0;
-    for (int k = 1; k <= kXcds; ++k) {
-      int cut = grid;
-      if (k < kXcds) {
-        const double target = total * k / kXcds;
-        double c = x.table_cost ? (double)x.table_cost[t] : 1.0;
-        while (t < n_tables - 1 && before + c * (double)wgs <= target) {
-          before += c * (double)wgs;
-          ++t;
-          c = x.table_cost ? (double)x.table_cost[t] : 1.0;
+    if (var_runs) {
+      // the same cut with runs whose size differs from table to table: a table's cost is its bags' cost
+      double all = 0.0;
+      for (int u = 0; u < n_tables; ++u) all += cost_of(u) * (double)n_bags;
+      for (int k = 1; k <= kXcds; ++k) {
+        int cut = grid;
+        if (k < kXcds) {
+          const double target = all * k / kXcds;
+          double c = cost_of(t);
+          while (t < n_tables - 1 && before + c * (double)n_bags <= target) {
+            before += c * (double)n_bags;
+            ++t;
+            c = cost_of(t);
+          }
+          const int64_t runs_t = L.run_start[t + 1] - L.run_start[t];
+          const int64_t within =
+              std::min<int64_t>(runs_t, std::max<int64_t>(0, (int64_t)((target - before) / (c * run_bags[t]) + 0.5)));
+          cut = (int)std::max<int64_t>(L.xcd_start[k - 1], (int64_t)L.run_start[t] + within);
         }
-        const int64_t within = std::min<int64_t>(wgs, std::max<int64_t>(0, (int64_t)((target - before) / c + 0.5)));
-        cut = (int)std::max<int64_t>(L.xcd_start[k - 1], (int64_t)t * wgs + within);
+        L.xcd_start[k] = cut;
+        longest = std::max(longest, cut - L.xcd_start[k - 1]);
       }
-      L.xcd_start[k] = cut;
-      longest = std::max(longest, cut - L.xcd_start[k - 1]);
+    } else {
+      for (int k = 1; k <= kXcds; ++k) {
+        int cut = grid;
+        if (k < kXcds) {
+          const double target = total * k / kXcds;
+          double c = cost_of(t);
+          while (t < n_tables - 1 && before + c * (double)wgs <= target) {
+            before += c * (double)wgs;
+            ++t;
+            c = cost_of(t);
+          }
+          const int64_t within = std::min<int64_t>(wgs, std::max<int64_t>(0, (int64_t)((target - before) / c + 0.5)));
+          cut = (int)std::max<int64_t>(L.xcd_start[k - 1], (int64_t)t * wgs + within);
+        }
+        L.xcd_start[k] = cut;
+        longest = std::max(longest, cut - L.xcd_start[k - 1]);
+      }
     }
     // Runs cut in four at the end of every segment (see the kernel): as many as a quarter of what an XCD holds
     // at once, and only in launches that fill the chip several times over.
     const int resident = device_cus() / kXcds * 6;  // workgroups of 256 lanes an XCD holds at the 6-per-CU occupancy
     L.tail_runs = 0;
-    if (block == kWG && L.bags_per_wg % 4 == 0 && L.bags_per_wg / 4 >= slots && longest >= 4 * resident)
-      L.tail_runs = FWDMI_BAG_TAIL_RUNS(resident);
+    bool can_cut = block == kWG && L.bags_per_wg % 4 == 0 && L.bags_per_wg / 4 >= slots;
+    for (int u = 0; var_runs && u < n_tables; ++u) can_cut = can_cut && run_bags[u] % 4 == 0 && run_bags[u] / 4 >= slots;
+    if (can_cut && longest >= 4 * resident) L.tail_runs = FWDMI_BAG_TAIL_RUNS(resident);
 #ifdef FWDMI_EXP_ENV
     if (const char* e = getenv("FWDMI_EXP_TAIL_RUNS")) L.tail_runs = atoi(e);
 #endif
@@ -1086,7 +1181,14 @@ int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_
   // every call on this GPU uses the same stream (or the caller orders them)
   if (const int rc = fwdmi_bag_tables_fill(tables_host, n_tables, dev_tables, stream)) return rc;
   fwdmi_bag_table none{};
-  return fwdmi::bag_dispatch(dev_tables, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, ext,
+  // the descriptors are on the host here: every table's own mean bag length comes with them
+  fwdmi_bag_ext with_len = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr};
+  float avg_len_t[fwdmi::kMaxVarTables];
+  if (!with_len.table_avg_len && n_tables <= fwdmi::kMaxVarTables && n_bags > 0) {
+    for (int32_t t = 0; t < n_tables; ++t) avg_len_t[t] = (float)((double)tables_host[t].input_size / (double)n_bags);
+    with_len.table_avg_len = avg_len_t;
+  }
+  return fwdmi::bag_dispatch(dev_tables, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, &with_len,
                              static_cast<hipStream_t>(stream));
 }
 

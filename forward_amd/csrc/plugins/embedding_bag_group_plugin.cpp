@@ -155,6 +155,8 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
   fwdmi_bag_table* const d_tables = static_cast<fwdmi_bag_table*>(workspace);
 
   int64_t n_off = -1, total_ids = 0;
+  constexpr int kMaxLenHints = 64;  // per-table mean bag lengths are a sizing hint for at most this many tables
+  float avg_len_t[kMaxLenHints];
   size_t row0 = 0;
   constexpr int kChunk = 64;
   fwdmi_bag_table chunk[kChunk];
@@ -174,6 +176,7 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
       n_off = no;
       if (ids.d[0] < 0) return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup::enqueue: negative id count");
       total_ids += ids.d[0];
+      if (t < kMaxLenHints) avg_len_t[t] = (float)ids.d[0];  // divided by the bag count below
       fwdmi_bag_table& d = chunk[k];
       d.data = static_cast<const char*>(d_data_) + row0 * (size_t)spec_.dim * es;
       d.input = inputs[per * t];
@@ -211,6 +214,10 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
   x.oob_flag = d_oob_;
   x.flags = (spec_.xcd_affinity ? FWDMI_BAG_XCD_TABLE_AFFINITY : 0) | (per == 3 ? FWDMI_BAG_TABLE_WEIGHTS : 0);
   x.table_cost = spec_.cost.data();
+  if (T <= kMaxLenHints) {
+    for (int t = 0; t < T; ++t) avg_len_t[t] /= (float)n_bags;
+    x.table_avg_len = avg_len_t;
+  }
   const double avg_len = (double)total_ids / ((double)n_bags * T);
   return fwdmi_embedding_bag_multi(d_tables, T, n_bags, outputs[0], spec_.dim, static_cast<int>(spec_.op), avg_len,
                                    &x, hipStream);

@@ -31,7 +31,8 @@ class BagExt(C.Structure):
     _fields_ = [("table_dtype", C.c_int32), ("index_dtype", C.c_int32), ("out_dtype", C.c_int32),
                 ("include_last_offset", C.c_int32), ("per_sample_weights", C.c_void_p),
                 ("max_indices", C.c_void_p), ("out_row_stride", C.c_int64), ("oob_flag", C.c_void_p),
-                ("flags", C.c_int32), ("table_cost", C.c_void_p), ("square_sum_out", C.c_void_p)]
+                ("flags", C.c_int32), ("table_cost", C.c_void_p), ("square_sum_out", C.c_void_p),
+                ("table_avg_len", C.c_void_p)]
 
 
 class EmbExt(C.Structure):

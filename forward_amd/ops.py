@@ -44,7 +44,7 @@ def _op(mode):
 
 
 def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_indices=None, out_row_stride=0,
-         oob_flag=None, flags=0, table_cost=None, square_sum_out=None):
+         oob_flag=None, flags=0, table_cost=None, square_sum_out=None, table_avg_len=None):
     x = lib.BagExt()
     x.table_dtype = _FDT[table.dtype]
     x.index_dtype = _IDT[indices.dtype]
@@ -57,6 +57,7 @@ def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_ind
     x.flags = flags
     x.table_cost = table_cost.ctypes.data if table_cost is not None else None
     x.square_sum_out = square_sum_out.data_ptr() if square_sum_out is not None else None
+    x.table_avg_len = table_avg_len.ctypes.data if table_avg_len is not None else None
     return x
 
 
@@ -174,6 +175,8 @@ class MultiTableBatch:
                        0 if w is None else w.data_ptr())
         self.width = max(out_cols) + self.dim
         self.total_indices = int(sum(i.numel() for i in self.indices))
+        # mean ids per bag of every table: tables that differ much in it get runs of their own size
+        self.table_avg_len = np.array([i.numel() / max(1, self.n_bags) for i in self.indices], np.float32)
         self.desc = torch.from_numpy(desc).to(self.tables[0].device)
 
     def default_table_cost(self):
@@ -198,7 +201,8 @@ class MultiTableBatch:
             _require(cost.shape == (self.n_tables,), 'cost.shape == (self.n_tables,)')
         x = _ext(self.tables[0], self.indices[0], odt, out_row_stride=out.shape[1], oob_flag=oob_flag,
                  flags=(lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0) |
-                       (lib.BAG_TABLE_WEIGHTS if self.weighted else 0), table_cost=cost)
+                       (lib.BAG_TABLE_WEIGHTS if self.weighted else 0), table_cost=cost,
+                 table_avg_len=self.table_avg_len)
         avg = self.total_indices / max(1, self.n_bags * self.n_tables)
         lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(self.desc), self.n_tables, self.n_bags, _p(out), self.dim,
                                                     _op(mode), avg, C.byref(x), _stream(stream)))
@@ -259,7 +263,8 @@ def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offse
     lib.check(lib.dll.fwdmi_bag_tables_fill(desc.ctypes.data, n, _p(d_desc), s))
     x = _ext(tables[0], indices[0], odt, include_last_offset=include_last_offset, out_row_stride=out.shape[1],
              oob_flag=oob_flag, flags=(lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0) |
-             (lib.BAG_TABLE_WEIGHTS if weighted else 0), table_cost=cost)
+             (lib.BAG_TABLE_WEIGHTS if weighted else 0), table_cost=cost,
+             table_avg_len=np.array([desc[t, 4] / max(1, n_bags) for t in range(n)], np.float32))
     lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(d_desc), n, n_bags, _p(out), dim, _op(mode),
                                                 total / max(1, n_bags * n), C.byref(x), s))
     return out

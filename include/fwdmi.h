@@ -95,6 +95,13 @@ typedef struct fwdmi_bag_ext {
                                   bag: the two reductions a factorisation-machine term needs
                                   (the reference builds them as two plugins over two copies of
                                   the table, source/fwd_tf/tf_cvt/tf_desc_creators/tf_embedding_bag_creator.h:43-95) */
+  const float* table_avg_len;  /* HOST array [n_tables] or NULL: mean ids per bag of each table of a
+                                  multi-table launch.  With it, a table's share of the XCD segments
+                                  (FWDMI_BAG_XCD_TABLE_AFFINITY) follows its bags' length as well as
+                                  table_cost, and in launches of at most 64 tables those whose means
+                                  differ by half or more get runs of their own size; without it every
+                                  table counts as avg_bag_len long.  A sizing hint only: results do
+                                  not depend on it */
 } fwdmi_bag_ext;
 
 /* Multi-table launches only: renumber workgroups so that each of the 8 XCDs (one L2 each)

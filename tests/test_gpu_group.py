@@ -269,8 +269,10 @@ def test_quarter_runs_at_segment_ends_on_ragged_tables(oracle, tdt, idt):
 @pytest.mark.parametrize("idt", [np.int32, np.int64])
 def test_tables_of_very_different_bag_lengths(oracle, idt):
     """One-hot tables beside tables of long bags in one launch: runs are sized from the mean bag
-    length of the whole launch, so a run of a long-bag table holds several times the ids the id
-    window takes and reads its ids unstaged.  With weights too; whole output against the oracle."""
+    length of the whole launch unless every table's own mean comes with the call
+    (``fwdmi_bag_ext.table_avg_len``: the tensor wrappers pass it), which gives the tables runs of
+    their own size and the XCDs shares by bag length.  Both ways, with weights too, through the
+    persistent descriptors and the per-call ones; whole output against the oracle."""
     from forward_amd import ops
     rng = np.random.Generator(np.random.PCG64(77))
     dim, n_bags = 64, 30000
@@ -298,3 +300,13 @@ def test_tables_of_very_different_bag_lengths(oracle, idt):
             got = batch.forward(out=torch.full((n_bags, len(rows) * dim), 3.0, dtype=torch.float16, device="cuda"),
                                 xcd_table_affinity=affinity)
             assert_bits_equal(host(got), want, "weights %s, affinity %s" % (weights is not None, affinity))
+            hints, batch.table_avg_len = batch.table_avg_len, None      # one run size for all tables
+            got = batch.forward(xcd_table_affinity=affinity)
+            batch.table_avg_len = hints
+            assert_bits_equal(host(got), want, "no length hints, weights %s, affinity %s" % (weights is not None, affinity))
+        got = ops.embedding_bag_group(d_tab, d_ids, d_off, per_sample_weights=None if weights is None else
+                                      [dev(w) for w in weights])
+        assert_bits_equal(host(got), want, "per-call descriptors, weights %s" % (weights is not None))
+    batch.table_avg_len = np.full(len(rows), -1.0, np.float32)
+    with pytest.raises(lib.FwdmiError, match="table_avg_len"):
+        batch.forward(xcd_table_affinity=True)

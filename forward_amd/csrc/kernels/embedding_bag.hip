@@ -818,7 +818,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
                  void* output, int64_t n_bags, int64_t fixed_len, int dim, int op, double avg_len,
                  const fwdmi_bag_ext* ext, hipStream_t stream) {
   clear_error();
-  static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr};
+  static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr};
   const fwdmi_bag_ext& x = ext ? *ext : kDefaultExt;
 
   if (!is_float_dtype(x.table_dtype) || !is_float_dtype(x.out_dtype) || !is_index_dtype(x.index_dtype))
@@ -1102,7 +1102,7 @@ int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t of
     return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "gather: batch %lld x %lld", (long long)batch_size,
                             (long long)offset);
   // A gather is a sum over bags of exactly one id.
-  fwdmi_bag_ext x = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr};
+  fwdmi_bag_ext x = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr};
   x.per_sample_weights = nullptr;
   x.max_indices = nullptr;
   x.square_sum_out = nullptr;

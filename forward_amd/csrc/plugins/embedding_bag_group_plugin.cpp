@@ -86,7 +86,7 @@ Dims EmbeddingBagGroupPlugin::getOutputDimensions(int outputIndex, const Dims* i
   }
   Dims out{};
   out.nbDims = 2;
-  out.d[0] = n_off - (spec_.opt.include_last_offset ? 1 : 0);
+  out.d[0] = (int32_t)(n_off - (spec_.opt.include_last_offset ? 1 : 0));
   out.d[1] = T * spec_.dim;
   return out;
 }

@@ -46,6 +46,7 @@ constexpr int kWG = 256;           // lanes per workgroup (large batches; small 
 constexpr int kIdxBytes = FWDMI_BAG_IDX_BYTES;   // LDS bytes of the id window per workgroup (4096 row numbers / 2048 64-bit ids)
 constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
 constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting sort
+constexpr int kInlineTables = FWDMI_BAG_INLINE_TABLES;  // table descriptors that travel with the launch as kernel arguments
 constexpr int kMaxVarTables = 64;  // tables of a launch whose runs may differ in size from table to table
 #ifndef FWDMI_BAG_UNROLL
 #define FWDMI_BAG_UNROLL 8
@@ -70,8 +71,9 @@ constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3, kMaxValue = 4, kSumSq = 5 };
 
 struct BagLaunch {
-  const fwdmi_bag_table* tables;  // device array, or nullptr -> `single`
-  fwdmi_bag_table single;
+  const fwdmi_bag_table* tables;  // device array of descriptors, or nullptr -> `inline_tables`
+  fwdmi_bag_table inline_tables[kInlineTables];  // a single-table launch uses [0]
+  int32_t multi;  // several tables (descriptors in `tables` or inline): weights come with the descriptors
   const void* psw;  // per-sample weights of the single-table form (a table of a batch carries its own)
   void* out;
   void* out2;  // kSumSq: the sums of squares, laid out like `out`
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
     T.out_col = tp->out_col;
     T.weights = tp->weights;
   } else {
-    T = L.single;
+    T = L.inline_tables[t];
   }
 
   const int G = 1 << L.log2_g;
@@ -200,8 +202,8 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   if (nb <= 0) return;  // a quarter beyond the table's last bag (uniform over the workgroup)
   const TI FWDMI_GLOBAL* __restrict__ ids = gconst<TI>(T.input);
   // per-sample weights: the launch's (single table) or the table's own; none = weight 1
-  const TW FWDMI_GLOBAL* __restrict__ psw = gconst<TW>(L.tables ? T.weights : L.psw);
-  const bool has_w = KIND == kWeighted && (L.tables ? T.weights : L.psw) != nullptr;  // uniform
+  const TW FWDMI_GLOBAL* __restrict__ psw = gconst<TW>(L.multi ? T.weights : L.psw);
+  const bool has_w = KIND == kWeighted && (L.multi ? T.weights : L.psw) != nullptr;  // uniform
 
   // ---- stage the run's offsets (clamped) ------------------------------------------------
   for (int i = tid; i <= nb; i += wg_lanes) {
@@ -749,6 +751,8 @@ int scratch_on_current_device(fwdmi_bag_table** out) {
   return FWDMI_OK;
 }
 
+static_assert(sizeof(BagLaunch) <= 4096, "kernel arguments are limited to 4 KiB");
+
 struct BagShape {
   int grid, block;
   size_t lds;
@@ -813,11 +817,14 @@ int next_pow2(int v) {
 }
 
 // Validates arguments, picks the lane mapping and launches.  `tables_dev` non-null selects the
-// multi-table form (then `single` is only used for host-side checks of shared fields).
-int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_bag_table& single,
+// multi-table form with descriptors in device memory, `tables_inline` (host, at most kInlineTables)
+// the one whose descriptors travel as kernel arguments; with neither, `single` is the table.
+int bag_dispatch(const fwdmi_bag_table* tables_dev, const fwdmi_bag_table* tables_inline, int n_tables,
+                 const fwdmi_bag_table& single,
                  void* output, int64_t n_bags, int64_t fixed_len, int dim, int op, double avg_len,
                  const fwdmi_bag_ext* ext, hipStream_t stream) {
   clear_error();
+  const bool multi = tables_dev || tables_inline;
   static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr};
   const fwdmi_bag_ext& x = ext ? *ext : kDefaultExt;
 
@@ -829,15 +836,15 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   // dim: a row's byte size and a run's (bag, slice) count stay far inside 32 bits
   FWDMI_REQUIRE(n_bags >= 0 && dim > 0 && dim <= (1 << 24) && n_tables > 0,
                 "embedding bag: n_bags=%lld dim=%d (1 .. 2^24) n_tables=%d", (long long)n_bags, dim, n_tables);
-  FWDMI_REQUIRE(!(x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS))) || op == FWDMI_OP_SUM,
+  FWDMI_REQUIRE(!(x.per_sample_weights || (multi && (x.flags & FWDMI_BAG_TABLE_WEIGHTS))) || op == FWDMI_OP_SUM,
                 "embedding bag: per_sample_weights needs op SUM (got %d)", op);
-  FWDMI_REQUIRE(!x.max_indices || (op == FWDMI_OP_MAX && !tables_dev),
+  FWDMI_REQUIRE(!x.max_indices || (op == FWDMI_OP_MAX && !multi),
                 "embedding bag: max_indices needs op MAX on a single table");
   const int64_t out_stride = x.out_row_stride > 0 ? x.out_row_stride : dim;
   FWDMI_REQUIRE(out_stride >= dim, "embedding bag: out_row_stride %lld < dim %d", (long long)out_stride, dim);
   if (n_bags == 0) return FWDMI_OK;
   FWDMI_REQUIRE(output != nullptr, "embedding bag: null output");
-  if (!tables_dev) {
+  if (!multi) {
     FWDMI_REQUIRE(single.count > 0 && single.data, "embedding bag: empty table");
     FWDMI_REQUIRE(single.input_size >= 0 && (single.input_size == 0 || single.input),
                   "embedding bag: null ids");
@@ -849,12 +856,19 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   const int vec_w = (int)(16 / sw);
   // 128-bit row loads need 16-byte row pitch and base; a multi-table launch is checked by its caller.
   bool vec = (dim % vec_w) == 0;
-  if (!tables_dev) vec = vec && (reinterpret_cast<uintptr_t>(single.data) % 16) == 0;
+  if (!multi) vec = vec && (reinterpret_cast<uintptr_t>(single.data) % 16) == 0;
   const int VEC = vec ? vec_w : 1;
 
   BagLaunch L{};
   L.tables = tables_dev;
-  L.single = single;
+  L.multi = multi;
+  if (tables_inline) {
+    FWDMI_REQUIRE(n_tables <= kInlineTables, "embedding bag: %d tables do not fit the launch's arguments (%d)", n_tables,
+                  kInlineTables);
+    std::copy(tables_inline, tables_inline + n_tables, L.inline_tables);
+  } else {
+    L.inline_tables[0] = single;
+  }
   L.out = output;
   L.max_indices = x.max_indices;
   L.out2 = x.square_sum_out;
@@ -880,7 +894,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   // launch cannot see its tables' sizes here; a run of such a table that does not fit the window
   // reads its ids from global memory.)
   const bool i64_ids = x.index_dtype == FWDMI_I64;
-  const bool wide_ids = i64_ids && !tables_dev &&
+  const bool wide_ids = i64_ids && !multi &&
                         (single.count > (1 << 24) || (uint64_t)single.count * dim * sw > ((uint64_t)1 << 32));
   const int max_cap = kIdxBytes / (wide_ids ? 8 : 4);
   const int64_t total_bags = n_bags * n_tables;
@@ -892,7 +906,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   while (block > 64 && block / 2 >= lanes && (int64_t)(block / 2 / lanes) >= want_bags * L.n_slices) block /= 2;
   const int slots = block / lanes;
   // Bags of a run and words of its id window for bags of `avg` ids on average.
-  const bool weighted_launch = x.per_sample_weights || (tables_dev && (x.flags & FWDMI_BAG_TABLE_WEIGHTS));
+  const bool weighted_launch = x.per_sample_weights || (multi && (x.flags & FWDMI_BAG_TABLE_WEIGHTS));
   auto size_run = [&](double avg, int64_t want, int* bags, int* cap) {
     // a whole number of rounds over the slots
     const int64_t units = std::max<int64_t>(slots, want * L.n_slices / slots * slots);
@@ -917,7 +931,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   // (28.6 M ids): 0.562 ms with one run size.
   int run_bags[kMaxVarTables];
   bool var_runs = false;
-  if (tables_dev && x.table_avg_len && n_tables > 1 && n_tables <= kMaxVarTables) {
+  if (multi && x.table_avg_len && n_tables > 1 && n_tables <= kMaxVarTables) {
     const int64_t want_all = std::min<int64_t>(std::max<int64_t>(1, total_bags / target_wgs), kMaxBagsPerWG);
     int lo = INT_MAX, hi = 0, cap_max = 0;
     for (int t = 0; t < n_tables; ++t) {
@@ -957,7 +971,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   L.vec_store = VEC > 1 && (reinterpret_cast<uintptr_t>(output) % store_align) == 0 &&
                 (reinterpret_cast<uintptr_t>(x.square_sum_out) % store_align) == 0 &&
                 ((out_stride * so) % store_align) == 0 &&
-                (tables_dev || (single.out_col * so) % store_align == 0);
+                (multi || (single.out_col * so) % store_align == 0);
 
   // A result of several MiB does not survive in the 4 MiB L2 of the XCD that wrote it until somebody
   // reads it (and a reader on another XCD would not find it there anyway); written with the
@@ -978,7 +992,7 @@ int bag_dispatch(const fwdmi_bag_table* tables_dev, int n_tables, const fwdmi_ba
   int grid = (int)total_runs;
   L.total_wgs = grid;
   L.xcd_affinity = 0;
-  if (tables_dev && n_tables > 1 && (x.flags & FWDMI_BAG_XCD_TABLE_AFFINITY)) {
+  if (multi && n_tables > 1 && (x.flags & FWDMI_BAG_XCD_TABLE_AFFINITY)) {
     // Cut the table-major work list into eight contiguous segments of equal estimated cost
     // (equal length when the caller gives no per-table cost).
     L.xcd_affinity = 1;
@@ -1081,7 +1095,7 @@ int fwdmi_embedding_bag(const void* input, const void* input_2, void* output, in
                         int64_t data_offset, int32_t op_type, const fwdmi_bag_ext* ext, void* stream) {
   fwdmi_bag_table t{data, input, input_2, count, input_size, data_offset, 0, nullptr};
   const double avg = block_size > 0 ? (double)input_size / (double)block_size : 1.0;
-  return fwdmi::bag_dispatch(nullptr, 1, t, output, block_size, -1, dim, op_type, avg, ext,
+  return fwdmi::bag_dispatch(nullptr, nullptr, 1, t, output, block_size, -1, dim, op_type, avg, ext,
                              static_cast<hipStream_t>(stream));
 }
 
@@ -1092,7 +1106,7 @@ int fwdmi_embedding_bag_fixed(const void* input, void* output, int64_t batch_siz
     return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "fixed-length bags: batch %lld x length %lld",
                             (long long)batch_size, (long long)offset);
   fwdmi_bag_table t{data, input, nullptr, count, batch_size * offset, data_offset, 0, nullptr};
-  return fwdmi::bag_dispatch(nullptr, 1, t, output, batch_size, offset, dim, op_type, (double)offset, ext,
+  return fwdmi::bag_dispatch(nullptr, nullptr, 1, t, output, batch_size, offset, dim, op_type, (double)offset, ext,
                              static_cast<hipStream_t>(stream));
 }
 
@@ -1109,7 +1123,7 @@ int fwdmi_gather(const void* input, void* output, int64_t batch_size, int64_t of
   x.out_row_stride = 0;
   const int64_t n = batch_size * offset;
   fwdmi_bag_table t{data, input, nullptr, count, n, data_offset, 0, nullptr};
-  return fwdmi::bag_dispatch(nullptr, 1, t, output, n, 1, dim, FWDMI_OP_SUM, 1.0, &x,
+  return fwdmi::bag_dispatch(nullptr, nullptr, 1, t, output, n, 1, dim, FWDMI_OP_SUM, 1.0, &x,
                              static_cast<hipStream_t>(stream));
 }
 
@@ -1122,7 +1136,7 @@ int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_table
                             "multi-table bags: per-sample weights go into the table descriptors "
                             "(FWDMI_BAG_TABLE_WEIGHTS), not into ext->per_sample_weights");
   fwdmi_bag_table none{};
-  return fwdmi::bag_dispatch(tables_dev, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, ext,
+  return fwdmi::bag_dispatch(tables_dev, nullptr, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, ext,
                              static_cast<hipStream_t>(stream));
 }
 
@@ -1142,12 +1156,72 @@ int fwdmi_bag_tables_fill(const fwdmi_bag_table* tables_host, int32_t n_tables, 
   return FWDMI_OK;
 }
 
+namespace {
+// What the device-descriptor form leaves to its caller, checked where the descriptors are host memory.
+int check_host_tables(const char* what, const fwdmi_bag_table* tables_host, int32_t n_tables, int32_t dim,
+                      const fwdmi_bag_ext* ext) {
+  const size_t sw = ext ? fwdmi::dtype_size(ext->table_dtype) : sizeof(float);
+  const size_t so = ext ? fwdmi::dtype_size(ext->out_dtype) : sizeof(float);
+  const int64_t stride = ext && ext->out_row_stride > 0 ? ext->out_row_stride : dim;
+  for (int32_t t = 0; t < n_tables; ++t) {
+    const fwdmi_bag_table& d = tables_host[t];
+    FWDMI_REQUIRE(d.count <= 0 || d.data, "%s: table %d has rows but no data", what, t);
+    FWDMI_REQUIRE(d.input_size >= 0 && (d.input_size == 0 || d.input) && d.input_2, "%s: table %d lacks ids or offsets", what, t);
+    FWDMI_REQUIRE(d.out_col >= 0 && dim > 0 && d.out_col + dim <= stride,
+                  "%s: table %d writes columns %lld.. beyond the row of %lld", what, t, (long long)d.out_col,
+                  (long long)stride);
+    if (sw && ((size_t)dim * sw) % 16 == 0) {  // rows are read (and written) as 16-byte slices
+      const size_t store_align = std::min<size_t>(16, 16 / sw * so);
+      FWDMI_REQUIRE(reinterpret_cast<uintptr_t>(d.data) % 16 == 0 && ((size_t)d.out_col * so) % store_align == 0,
+                    "%s: table %d: data or output column not aligned to its slices", what, t);
+    }
+  }
+  return FWDMI_OK;
+}
+
+// Every table's own mean bag length, from host descriptors, unless the caller gave them.
+void fill_avg_len(fwdmi_bag_ext* x, float* avg_len_t, const fwdmi_bag_table* tables_host, int32_t n_tables,
+                  int64_t n_bags) {
+  if (x->table_avg_len || n_tables > fwdmi::kMaxVarTables || n_bags <= 0) return;
+  for (int32_t t = 0; t < n_tables; ++t) avg_len_t[t] = (float)((double)tables_host[t].input_size / (double)n_bags);
+  x->table_avg_len = avg_len_t;
+}
+
+const fwdmi_bag_ext kPlainExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr};
+}  // namespace
+
+int fwdmi_embedding_bag_multi_host(const fwdmi_bag_table* tables_host, int32_t n_tables, fwdmi_bag_table* tables_dev,
+                                   int64_t n_bags, void* output, int32_t dim, int32_t op_type, double avg_bag_len,
+                                   const fwdmi_bag_ext* ext, void* stream) {
+  fwdmi::clear_error();
+  static const char* const kWhat = "multi-table bags (host descriptors)";
+  if (!tables_host || n_tables <= 0) return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "%s: null or empty table array", kWhat);
+  if (ext && ext->per_sample_weights)
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG,
+                            "multi-table bags: per-sample weights go into the table descriptors "
+                            "(FWDMI_BAG_TABLE_WEIGHTS), not into ext->per_sample_weights");
+  if (const int rc = check_host_tables(kWhat, tables_host, n_tables, dim, ext)) return rc;
+  fwdmi_bag_ext x = ext ? *ext : kPlainExt;
+  float avg_len_t[fwdmi::kMaxVarTables];
+  fill_avg_len(&x, avg_len_t, tables_host, n_tables, n_bags);
+  fwdmi_bag_table none{};
+  if (n_tables <= fwdmi::kInlineTables)  // the descriptors are part of the launch: no second launch, no device array
+    return fwdmi::bag_dispatch(nullptr, tables_host, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, &x,
+                               static_cast<hipStream_t>(stream));
+  if (!tables_dev)
+    return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "%s: %d tables need a device array for their descriptors (more than %d)",
+                            kWhat, n_tables, fwdmi::kInlineTables);
+  if (const int rc = fwdmi_bag_tables_fill(tables_host, n_tables, tables_dev, stream)) return rc;
+  return fwdmi::bag_dispatch(tables_dev, nullptr, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, &x,
+                             static_cast<hipStream_t>(stream));
+}
+
 int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_t n_tables, int64_t n_bags,
                                       void* output, int32_t dim, int32_t op_type, double avg_bag_len,
                                       const fwdmi_bag_ext* ext, void* stream) {
   fwdmi::clear_error();
-  if (!tables_host || n_tables <= 0)
-    return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "multi-table bags (no allocation): null or empty table array");
+  static const char* const kWhat = "multi-table bags (no allocation)";
+  if (!tables_host || n_tables <= 0) return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "%s: null or empty table array", kWhat);
   if (n_tables > fwdmi::kNoAllocMaxTables)
     return fwdmi::set_error(FWDMI_ERR_BAD_ARG,
                             "multi-table bags (no allocation): %d tables exceed the built-in descriptor "
@@ -1158,23 +1232,7 @@ int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_
                             "multi-table bags: per-sample weights go into the table descriptors "
                             "(FWDMI_BAG_TABLE_WEIGHTS), not into ext->per_sample_weights");
   // the descriptors are host memory here, so what the device form leaves to its caller is checked
-  const size_t sw = ext ? fwdmi::dtype_size(ext->table_dtype) : sizeof(float);
-  const size_t so = ext ? fwdmi::dtype_size(ext->out_dtype) : sizeof(float);
-  const int64_t stride = ext && ext->out_row_stride > 0 ? ext->out_row_stride : dim;
-  for (int32_t t = 0; t < n_tables; ++t) {
-    const fwdmi_bag_table& d = tables_host[t];
-    FWDMI_REQUIRE(d.count <= 0 || d.data, "multi-table bags (no allocation): table %d has rows but no data", t);
-    FWDMI_REQUIRE(d.input_size >= 0 && (d.input_size == 0 || d.input) && d.input_2,
-                  "multi-table bags (no allocation): table %d lacks ids or offsets", t);
-    FWDMI_REQUIRE(d.out_col >= 0 && dim > 0 && d.out_col + dim <= stride,
-                  "multi-table bags (no allocation): table %d writes columns %lld.. beyond the row of %lld", t,
-                  (long long)d.out_col, (long long)stride);
-    if (sw && ((size_t)dim * sw) % 16 == 0) {  // rows are read (and written) as 16-byte slices
-      const size_t store_align = std::min<size_t>(16, 16 / sw * so);
-      FWDMI_REQUIRE(reinterpret_cast<uintptr_t>(d.data) % 16 == 0 && ((size_t)d.out_col * so) % store_align == 0,
-                    "multi-table bags (no allocation): table %d: data or output column not aligned to its slices", t);
-    }
-  }
+  if (const int rc = check_host_tables(kWhat, tables_host, n_tables, dim, ext)) return rc;
   fwdmi_bag_table* dev_tables = nullptr;
   if (const int rc = fwdmi::scratch_on_current_device(&dev_tables)) return rc;
   // stream order keeps a call's descriptors intact until its launch has read them, as long as
@@ -1182,13 +1240,10 @@ int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_
   if (const int rc = fwdmi_bag_tables_fill(tables_host, n_tables, dev_tables, stream)) return rc;
   fwdmi_bag_table none{};
   // the descriptors are on the host here: every table's own mean bag length comes with them
-  fwdmi_bag_ext with_len = ext ? *ext : fwdmi_bag_ext{FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr};
+  fwdmi_bag_ext with_len = ext ? *ext : kPlainExt;
   float avg_len_t[fwdmi::kMaxVarTables];
-  if (!with_len.table_avg_len && n_tables <= fwdmi::kMaxVarTables && n_bags > 0) {
-    for (int32_t t = 0; t < n_tables; ++t) avg_len_t[t] = (float)((double)tables_host[t].input_size / (double)n_bags);
-    with_len.table_avg_len = avg_len_t;
-  }
-  return fwdmi::bag_dispatch(dev_tables, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, &with_len,
+  fill_avg_len(&with_len, avg_len_t, tables_host, n_tables, n_bags);
+  return fwdmi::bag_dispatch(dev_tables, nullptr, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, &with_len,
                              static_cast<hipStream_t>(stream));
 }
 

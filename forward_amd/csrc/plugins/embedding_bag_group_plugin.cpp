@@ -138,8 +138,10 @@ void EmbeddingBagGroupPlugin::terminate() noexcept {
   initialized_ = false;
 }
 
-// Writes this call's table descriptors into the workspace (as kernel arguments, so nothing is
-// staged on the host and the call stays stream-ordered), then reduces all tables in one launch.
+// Reduces all tables in one launch.  This call's table descriptors travel with that launch as
+// kernel arguments (up to FWDMI_BAG_INLINE_TABLES tables) or are written into the workspace by
+// small launches before it (more tables); either way nothing is staged on the host and the call
+// stays stream-ordered.
 int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const PluginTensorDesc* outputDesc,
                                      const void* const* inputs, void* const* outputs, void* workspace,
                                      void* hipStream) noexcept {
@@ -159,6 +161,7 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
   float avg_len_t[kMaxLenHints];
   size_t row0 = 0;
   constexpr int kChunk = 64;
+  static_assert(kChunk >= FWDMI_BAG_INLINE_TABLES, "one chunk holds every table of the inline form");
   fwdmi_bag_table chunk[kChunk];
   for (int t0 = 0; t0 < T; t0 += kChunk) {
     const int n = std::min(kChunk, T - t0);
@@ -198,8 +201,10 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
       if (!d.input_2) return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup::enqueue: null offsets (table %d)", t);
       row0 += (size_t)spec_.count[t];
     }
-    const int rc = fwdmi_bag_tables_fill(chunk, n, d_tables + t0, hipStream);
-    if (rc != FWDMI_OK) return rc;
+    if (T > FWDMI_BAG_INLINE_TABLES) {  // fewer travel with the launch itself (below)
+      const int rc = fwdmi_bag_tables_fill(chunk, n, d_tables + t0, hipStream);
+      if (rc != FWDMI_OK) return rc;
+    }
   }
   const int64_t n_bags = n_off - (spec_.opt.include_last_offset ? 1 : 0);
   if (n_bags < 0) return set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBagGroup::enqueue: offsets input is empty");
@@ -219,6 +224,9 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
     x.table_avg_len = avg_len_t;
   }
   const double avg_len = (double)total_ids / ((double)n_bags * T);
+  if (T <= FWDMI_BAG_INLINE_TABLES)  // `chunk` holds them all: the descriptors are kernel arguments of the one launch
+    return fwdmi_embedding_bag_multi_host(chunk, T, nullptr, n_bags, outputs[0], spec_.dim, static_cast<int>(spec_.op),
+                                          avg_len, &x, hipStream);
   return fwdmi_embedding_bag_multi(d_tables, T, n_bags, outputs[0], spec_.dim, static_cast<int>(spec_.op), avg_len,
                                    &x, hipStream);
 }

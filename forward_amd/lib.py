@@ -25,6 +25,7 @@ FORMAT_LINEAR = 0
 OP_SUM, OP_MEAN, OP_MAX, OP_SQUARE_SUM, OP_GATHER = 0, 1, 2, 3, 999
 BAG_XCD_TABLE_AFFINITY = 1
 BAG_TABLE_WEIGHTS = 2
+BAG_INLINE_TABLES = 40        # FWDMI_BAG_INLINE_TABLES
 
 
 class BagExt(C.Structure):
@@ -89,6 +90,8 @@ SIGNATURES = {
     "fwdmi_bag_table_cost": (C.c_int, [_vp, _i32, _vp]),
     "fwdmi_bag_tables_fill": (C.c_int, [_vp, _i32, _vp, _vp]),
     "fwdmi_embedding_bag_multi": (C.c_int, [_vp, _i32, _i64, _vp, _i32, _i32, C.c_double, C.POINTER(BagExt), _vp]),
+    "fwdmi_embedding_bag_multi_host": (C.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _i32, C.c_double, C.POINTER(BagExt),
+                                                 _vp]),
     "fwdmi_embedding_bag_multi_noalloc": (C.c_int, [_vp, _i32, _i64, _vp, _i32, _i32, C.c_double, C.POINTER(BagExt),
                                                     _vp]),
     "fwdmi_layer_norm": (C.c_int, [_vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _i32, C.c_float]),

@@ -214,8 +214,8 @@ def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offse
     """All tables of a sparse stage in one launch with this call's ids / offsets:
     ``[n_bags, T*dim]``, columns ``t*dim ..`` equal to ``embedding_bag(tables[t], indices[t], offsets[t])``.
 
-    The table descriptors go to a device buffer as kernel arguments on torch's current stream
-    (``fwdmi_bag_tables_fill``), so nothing is staged or synchronised on the host.
+    The table descriptors travel as kernel arguments on torch's current stream (with the launch itself,
+    or for many tables through ``fwdmi_bag_tables_fill``), so nothing is staged or synchronised on the host.
     """
     n = len(tables)
     _require(n > 0 and len(indices) == n and len(offsets) == n, 'len(tables) == len(indices) == len(offsets) > 0')
@@ -258,15 +258,15 @@ def embedding_bag_group(tables, indices, offsets, mode="sum", include_last_offse
         else:
             cost = np.ascontiguousarray(table_cost, np.float32)
             _require(cost.shape == (n,), 'table_cost has one entry per table')
-    d_desc = torch.empty(n * 64, dtype=torch.uint8, device=tables[0].device)
     s = _stream(None)
-    lib.check(lib.dll.fwdmi_bag_tables_fill(desc.ctypes.data, n, _p(d_desc), s))
     x = _ext(tables[0], indices[0], odt, include_last_offset=include_last_offset, out_row_stride=out.shape[1],
              oob_flag=oob_flag, flags=(lib.BAG_XCD_TABLE_AFFINITY if xcd_table_affinity else 0) |
-             (lib.BAG_TABLE_WEIGHTS if weighted else 0), table_cost=cost,
-             table_avg_len=np.array([desc[t, 4] / max(1, n_bags) for t in range(n)], np.float32))
-    lib.check(lib.dll.fwdmi_embedding_bag_multi(_p(d_desc), n, n_bags, _p(out), dim, _op(mode),
-                                                total / max(1, n_bags * n), C.byref(x), s))
+             (lib.BAG_TABLE_WEIGHTS if weighted else 0), table_cost=cost)
+    # up to lib.BAG_INLINE_TABLES descriptors travel with the launch as kernel arguments; more need a device array
+    d_desc = None if n <= lib.BAG_INLINE_TABLES else torch.empty(n * 64, dtype=torch.uint8, device=tables[0].device)
+    lib.check(lib.dll.fwdmi_embedding_bag_multi_host(desc.ctypes.data, n, _p(d_desc),
+                                                     n_bags, _p(out), dim, _op(mode), total / max(1, n_bags * n),
+                                                     C.byref(x), s))
     return out
 
 

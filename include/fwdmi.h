@@ -179,6 +179,21 @@ int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_table
                               const fwdmi_bag_ext* ext, void* stream);
 
 /*
+ * fwdmi_embedding_bag_multi for callers that hold the descriptors in HOST memory and rebuild them per
+ * call (a plugin's enqueue: new id / offset buffers every time).  Up to FWDMI_BAG_INLINE_TABLES tables travel with the launch
+ * itself, as kernel arguments: one launch, nothing staged, `tables_dev` is not used and may be NULL.
+ * More tables are written to `tables_dev` (a device array of n_tables descriptors, required then) by
+ * fwdmi_bag_tables_fill on the same stream first.  The descriptors are checked on the host (data /
+ * ids / offsets present, column block inside the output row, 16-byte alignment where rows are read as
+ * slices) and every table's mean bag length is taken from them unless ext->table_avg_len is given.
+ * Results equal those of fwdmi_embedding_bag_multi bit for bit.
+ */
+#define FWDMI_BAG_INLINE_TABLES 40
+int fwdmi_embedding_bag_multi_host(const fwdmi_bag_table* tables_host, int32_t n_tables, fwdmi_bag_table* tables_dev,
+                                   int64_t n_bags, void* output, int32_t dim, int32_t op_type, double avg_bag_len,
+                                   const fwdmi_bag_ext* ext, void* stream);
+
+/*
  * fwdmi_embedding_bag_multi for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
  * reference.  The descriptors are given in HOST memory; the library copies them (as kernel

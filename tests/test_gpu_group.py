@@ -310,3 +310,49 @@ def test_tables_of_very_different_bag_lengths(oracle, idt):
     batch.table_avg_len = np.full(len(rows), -1.0, np.float32)
     with pytest.raises(lib.FwdmiError, match="table_avg_len"):
         batch.forward(xcd_table_affinity=True)
+
+
+def test_host_descriptor_entry_point_limits(oracle):
+    """fwdmi_embedding_bag_multi_host: up to FWDMI_BAG_INLINE_TABLES tables need no device array for their
+    descriptors, more do; descriptors are checked on the host before anything is launched."""
+    import ctypes as C
+    from forward_amd import ops
+    rng = np.random.Generator(np.random.PCG64(31))
+    dim, n_bags = 32, 50
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def call(n, d_desc, mutate=None):
+        tables = [(rng.standard_normal((20 + t, dim)) * 0.3).astype(np.float32) for t in range(n)]
+        ids, offs = random_batch(rng, [t.shape[0] for t in tables], n_bags, np.int32, max_len=5)
+        keep = [dev(x) for x in tables + ids + offs]
+        desc = np.zeros((n, 8), np.int64)
+        for t in range(n):
+            desc[t] = (keep[t].data_ptr(), keep[n + t].data_ptr(), keep[2 * n + t].data_ptr(), tables[t].shape[0],
+                       ids[t].size, 0, t * dim, 0)
+        if mutate:
+            mutate(desc)
+        out = torch.full((n_bags, n * dim), 9.0, dtype=torch.float32, device="cuda")
+        x = ops._ext(keep[0], keep[n], torch.float32, out_row_stride=n * dim)
+        rc = lib.dll.fwdmi_embedding_bag_multi_host(desc.ctypes.data, n, C.c_void_p(d_desc.data_ptr() if d_desc is not None else 0),
+                                                    n_bags, C.c_void_p(out.data_ptr()), dim, 0, 2.0, C.byref(x), stream)
+        return rc, host(out), tables, ids, offs
+
+    for n, with_array in ((lib.BAG_INLINE_TABLES, False), (lib.BAG_INLINE_TABLES + 1, True)):
+        d_desc = torch.empty(n * 64, dtype=torch.uint8, device="cuda") if with_array else None
+        rc, got, tables, ids, offs = call(n, d_desc)
+        assert rc == 0, lib.last_error()
+        for t in (0, n // 2, n - 1):
+            want, _, _ = oracle.embedding_bag(tables[t], ids[t], offs[t], 0)
+            assert_bits_equal(got[:, t * dim:(t + 1) * dim], want, "%d tables, table %d" % (n, t))
+    rc, got, *_ = call(lib.BAG_INLINE_TABLES + 1, None)
+    assert rc == lib.ERR_BAD_ARG and "device array" in lib.last_error() and (got == 9.0).all()
+
+    def col_beyond_row(desc):
+        desc[1, 6] = 3 * dim
+    rc, got, *_ = call(3, None, col_beyond_row)
+    assert rc == lib.ERR_BAD_ARG and "beyond the row" in lib.last_error() and (got == 9.0).all()
+
+    def no_offsets(desc):
+        desc[2, 2] = 0
+    rc, got, *_ = call(3, None, no_offsets)
+    assert rc == lib.ERR_BAD_ARG and "offsets" in lib.last_error() and (got == 9.0).all()

@@ -1,8 +1,10 @@
 """The C-ABI library loads without a GPU and exports exactly what include/fwdmi.h declares."""
+import os
 import re
 import subprocess
 
 import numpy as np
+import pytest
 
 from forward_amd import lib
 
@@ -67,3 +69,19 @@ def test_table_cost_estimate():
     assert cost[0] == 1.0 and cost[1] == 1.0 and cost[3] == cost[4] and 1.0 < cost[2] < cost[3] < 2.0
     np.testing.assert_allclose(cost[2], 1.0 + 0.45 * 0.5, rtol=1e-6)    # 32 MiB is half way in log size
     assert lib.dll.fwdmi_bag_table_cost(None, 5, cost.ctypes.data) == lib.ERR_BAD_ARG
+
+
+def test_c_header_is_plain_c(tmp_path):
+    """include/fwdmi.h is what a C host (cgo, JNI glue, plain C) includes: it must compile as C99."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "fwdmi.h"\n'
+                   'int main(void) { fwdmi_bag_ext e = {0}; fwdmi_bag_table t = {0}; (void)e; (void)t;\n'
+                   '  return FWDMI_BAG_INLINE_TABLES > 0 && FWDMI_OP_SUM == 0 ? 0 : 1; }\n')
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    p = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, "-fsyntax-only", str(src)],
+                       capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr

@@ -529,6 +529,39 @@ def sweep_layer_norm(torch, ops):
                     rows, ld, "f16" if tdt == torch.float16 else "f32", ms, nbytes / ms / 1e6, tms, tms / ms), flush=True)
 
 
+def mixed_bag_lengths(torch, ops, workloads, wl, tabs):
+    """The workload's tables with every other table one-hot (one id per bag) and the rest with bags twice
+    as long (Zipf lengths 2 .. 200, mean 32.6), ids Zipf(1.1) as in the workload: the fused launch with
+    and without each table's own mean bag length (fwdmi_bag_ext.table_avg_len), checked equal."""
+    rng = np.random.Generator(np.random.PCG64(4005))
+    cdf = workloads.zipf_cdf(100, 1.1)
+    idx, off, n_ids = [], [], 0
+    for t in range(len(tabs)):
+        if t % 2 == 0:
+            lengths = np.ones(wl.n_bags, np.int64)
+        else:
+            lengths = 2 * (workloads.zipf_ranks(rng, 100, 1.1, wl.n_bags, cdf).astype(np.int64) + 1)
+        n = int(lengths.sum())
+        n_ids += n
+        ids = workloads.scatter_ranks(workloads.zipf_ranks(rng, wl.rows[t], 1.1, n), wl.rows[t]).astype(np.int32)
+        idx.append(torch.from_numpy(ids).cuda())
+        off.append(torch.from_numpy(workloads.offsets_from_lengths(lengths, np.int32)).cuda())
+    b = ops.MultiTableBatch(tabs, idx, off)
+    out = torch.empty((wl.n_bags, len(tabs) * wl.dim), dtype=tabs[0].dtype, device="cuda")
+    res = {"what": "every other table one-hot, the others Zipf lengths 2 .. 200 (mean 32.6); ids Zipf(1.1)",
+           "total_ids": n_ids, "bags": wl.n_bags * len(tabs)}
+    _, per = time_events(torch, lambda: b.forward(out=out, xcd_table_affinity=True), 40, 10)
+    res["ms_per_launch"] = float(per.mean())
+    res["bags_per_s"] = wl.n_bags * len(tabs) / (float(per.mean()) * 1e-3)
+    with_hints = out.clone()
+    hints, b.table_avg_len = b.table_avg_len, None
+    _, per = time_events(torch, lambda: b.forward(out=out, xcd_table_affinity=True), 40, 10)
+    b.table_avg_len = hints
+    res["ms_per_launch_without_table_avg_len"] = float(per.mean())
+    res["results_equal"] = bool(torch.equal(out.view(torch.int16), with_hints.view(torch.int16)))
+    return res
+
+
 def replay_times(torch, ops, wl, tabs, idx, off, steps=60):
     """Times (ms, median of HIP-event durations) of forward_amd/csrc/microbench/replay_gather.hip on the
     workload's id stream: the rows alone, the rows plus as many stored bytes as the product writes
@@ -802,6 +835,13 @@ def main():
                 result["replay_without_bags"] = rt
         except Exception as e:  # noqa: BLE001
             result["replay_without_bags"] = {"error": repr(e)}
+    if not args.no_extra and full:
+        # the same 26 tables with bag lengths that differ from table to table (one-hot features beside
+        # multi-hot ones): not the headline workload, reported for the launch's run sizing by table
+        try:
+            result["mixed_bag_lengths"] = mixed_bag_lengths(torch, ops, workloads, wl, tabs)
+        except Exception as e:  # noqa: BLE001
+            result["mixed_bag_lengths"] = {"error": repr(e)}
     if not args.no_extra:
         del tabs, batch
         result["extra"] = extra_measurements(torch, ops, workloads, max(10, args.steps), with_cpu=not args.no_cpu)

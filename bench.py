@@ -1,23 +1,26 @@
 #!/usr/bin/env python3
 """Benchmark of the embedding-side hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K (200)] [--warmup W (20)] [--prewarm P (300)] [--workload config4]
-                  [--no-cpu] [--no-extra]
+  python bench.py [--gpus 1] [--steps K (200)] [--warmup W (20)] [--prewarm P (300)] [--batches B (8)]
+                  [--workload config4] [--no-cpu] [--no-extra]
 
 A step is one pass of the DLRM-style sparse stage (BASELINE config 4): 26 sum-mode tables, fp16
 rows of dim 128, 65536 bags per table with truncated-Zipf lengths, Zipf ids, fp16 output
 concatenated to [65536, 3328], issued as ONE fused launch.  Inputs are resident in HBM before the
-timed region.  Prints one JSON line: bags/s over the whole job, the roofline position of the
-kernel from HIP-event timing of the same launches (time floor / kernel time, the floor being the
-larger of "measured bytes beyond L2 at the HBM peak" and "algorithmic bytes at the L1 return
-rate"), and a CPU baseline: libtorch CPU (the path the reference's unit tests compare against) at
-all host threads this process may use, with the C oracle port beside it.
+timed region; the steps cycle through B batches of fresh ids and bag lengths over the same tables
+(a serving loop never sees the same ids twice), the same-batch figure is reported beside it.
+Prints one JSON line: bags/s over the whole job, the roofline block of the kernel from HIP-event
+timing of the same launches (frac = algorithmic bytes / kernel time / HBM peak, which exceeds 1
+when caches serve most rows; frac_hbm_side = bytes counted beyond L2 / kernel time / HBM peak), and a
+CPU baseline: libtorch CPU (the path the reference's unit tests compare against) at all host
+threads this process may use, with the C oracle port beside it.
 
-  python bench.py --record-traffic FETCH_CSV WRITE_CSV
+  python bench.py --record-traffic FETCH_CSV WRITE_CSV [--batches B]
       (no GPU) turns two rocprofv3 --pmc counter_collection CSVs of
-      `bench.py --steps 3 --warmup 1 --prewarm 0 --no-cpu --no-extra --copy-calibration`
-      (FETCH_SIZE in one run, WRITE_SIZE in the other) into profiles/traffic.json, stamped with the
-      hash of the kernel sources they were measured on.
+      `bench.py --steps 16 --warmup 0 --prewarm 0 --batches B --no-cpu --no-extra --copy-calibration`
+      (FETCH_SIZE in one run, WRITE_SIZE in the other) into profiles/traffic.json (section
+      "rotating_batches" for B > 1, "same_batch" for B = 1), stamped with the hash of the kernel
+      sources they were measured on.
 """
 import argparse
 import hashlib
@@ -33,8 +36,8 @@ MI355X_PEAK_CLOCK_HZ = 2.4e9    # published peak engine clock
 ROOT = os.path.dirname(os.path.abspath(__file__))
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
 # the sources the 26-table kernel is compiled from: counter figures belong to one state of them
-KERNEL_SOURCES = ("forward_amd/csrc/kernels/embedding_bag.hip", "forward_amd/csrc/kernels/device_util.h",
-                  "forward_amd/csrc/common.h")
+KERNEL_SOURCES = ("forward_amd/csrc/kernels/embedding_bag.hip", "forward_amd/csrc/kernels/bag_plan.h",
+                  "forward_amd/csrc/kernels/bag_plan.cpp", "forward_amd/csrc/kernels/device_util.h")
 
 
 def log(*a):
@@ -49,6 +52,9 @@ def parse():
     ap.add_argument("--prewarm", type=int, default=300,
                     help="untimed launches before the warm-up steps, so that a short run (--steps 20 --warmup 5) is "
                          "timed at the steady engine clock like a long one; reported as prewarm_launches")
+    ap.add_argument("--batches", type=int, default=8,
+                    help="batches of fresh ids / bag lengths (same tables) the steps cycle through; 1 = every step "
+                         "replays the same batch")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU: write profiles/traffic.json from two rocprofv3 --pmc counter_collection CSVs")
     ap.add_argument("--workload", default="config4", choices=["config4"])
@@ -72,6 +78,9 @@ def parse():
     ap.add_argument("--lru-sim", action="store_true",
                     help="no GPU: rows fetched by an LRU cache of one XCD's L2 size over each table's id stream "
                          "(the floor of the re-fetch ratio for table-at-a-time processing)")
+    ap.add_argument("--hbm-gather", action="store_true",
+                    help="instead of the benchmark: uniform random ids over one 4 GiB fp16 table of dim 128 (far beyond "
+                         "every cache), the gather rate that is HBM and nothing else (one JSON line on stdout)")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the benchmark: single-table bag reduction over row widths, table types and "
                          "bag lengths with uniform random ids beside torch's GPU embedding_bag, then SkipLayerNorm "
@@ -103,9 +112,10 @@ def kernel_source_hash():
     return h.hexdigest()
 
 
-def load_traffic():
-    """HBM-side bytes per launch of the default workload from profiles/traffic.json, or None (with
-    a warning) when the file is absent or was measured on other kernel sources than the tree holds."""
+def load_traffic(section):
+    """HBM-side bytes per launch of the default workload from profiles/traffic.json (`section`:
+    "rotating_batches" or "same_batch"), or None (with a warning) when the file or the section is
+    absent or was measured on other kernel sources than the tree holds."""
     if not os.path.exists(TRAFFIC_JSON):
         log("warning: %s is absent: roofline.traffic is null" % TRAFFIC_JSON)
         return None
@@ -116,13 +126,18 @@ def load_traffic():
             "roofline.traffic is null until the counters are collected again (bench.py --record-traffic)"
             % (str(t.get("kernel_source_sha256"))[:12], kernel_source_hash()[:12]))
         return None
-    return t
+    if section not in t:
+        log("warning: profiles/traffic.json has no %s section: roofline.traffic is null" % section)
+        return None
+    return dict(t[section], kernel_source_sha256=t["kernel_source_sha256"])
 
 
-def record_traffic(fetch_csv, write_csv):
+def record_traffic(fetch_csv, write_csv, batches):
     """profiles/traffic.json from two rocprofv3 counter CSVs (FETCH_SIZE / WRITE_SIZE, KiB per
     dispatch).  Each counter is scaled by what it reads for the 1 GiB device copy of the same run
-    (--copy-calibration: 1 048 576 KiB read and as many written)."""
+    (--copy-calibration: 1 048 576 KiB read and as many written).  The counters sit at the L2's
+    far side (requests from L2 to the fabric): bytes the memory-side cache serves are counted like
+    bytes from DRAM."""
     import csv
 
     def per_kernel(path, counter):
@@ -149,19 +164,28 @@ def record_traffic(fetch_csv, write_csv):
     ws = kib / write_cal if write_cal else 1.0
     # the counters come in two granularities (32- and 64-byte units): snap the measured factor
     fs, ws = (min((1.0, 2.0, 4.0), key=lambda c: abs(c - x)) for x in (fs, ws))
-    out = {
-        "_comment": "HBM-side bytes per launch of bench.py's default workload from rocprofv3 --pmc FETCH_SIZE / "
-                    "WRITE_SIZE (KiB per dispatch), each scaled by what the counter reads for a 1 GiB device copy "
-                    "of the same run; written by bench.py --record-traffic",
-        "kernel_source_sha256": kernel_source_hash(), "kernel_source_files": list(KERNEL_SOURCES),
+    sec = {
+        "batches": batches,
         "fetch_size_kib_raw": fetch, "write_size_kib_raw": write, "dispatches": [nf, nw],
         "fetch_size_copy_kib_raw": fetch_cal, "write_size_copy_kib_raw": write_cal,
         "fetch_size_scale": fs, "write_size_scale": ws,
-        "bag_reduce_config4_fetch_bytes": int(round(fetch * fs * 1024)),
-        "bag_reduce_config4_write_bytes": int(round(write * ws * 1024)),
+        "fetch_bytes": int(round(fetch * fs * 1024)), "write_bytes": int(round(write * ws * 1024)),
     }
-    out["bag_reduce_config4_bytes_per_launch"] = (out["bag_reduce_config4_fetch_bytes"] +
-                                                  out["bag_reduce_config4_write_bytes"])
+    sec["bytes_per_launch"] = sec["fetch_bytes"] + sec["write_bytes"]
+    out = {}
+    if os.path.exists(TRAFFIC_JSON):
+        with open(TRAFFIC_JSON) as f:
+            out = json.load(f)
+        if out.get("kernel_source_sha256") != kernel_source_hash():
+            out = {}           # figures of another state of the kernel: nothing of them is kept
+    out["_comment"] = ("bytes per launch of bench.py's default workload beyond L2 (requests from L2 to the fabric: "
+                       "memory-side-cache hits count like DRAM reads) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                       "(KiB per dispatch), each scaled by what the counter reads for a 1 GiB device copy of the same "
+                       "run; rotating_batches: the steps cycle through fresh id batches, same_batch: every step "
+                       "replays one batch; written by bench.py --record-traffic")
+    out["kernel_source_sha256"] = kernel_source_hash()
+    out["kernel_source_files"] = list(KERNEL_SOURCES)
+    out["rotating_batches" if batches > 1 else "same_batch"] = sec
     with open(TRAFFIC_JSON, "w") as f:
         json.dump(out, f, indent=1)
         f.write("\n")
@@ -401,6 +425,63 @@ def plugin_level(torch, wl, tabs, idx, off, want):
     return res
 
 
+def microbench_dll():
+    """bench_aux/libfwdmi_microbench.so (the measurement aids), or None when it is not built."""
+    import ctypes as C
+    path = os.path.join(ROOT, "bench_aux", "libfwdmi_microbench.so")
+    return C.CDLL(path) if os.path.exists(path) else None
+
+
+def launch_floor_ms(torch, grid=1024, block=256):
+    """GPU time per launch of a kernel that does nothing, with the grid of the short launches (1024
+    workgroups of 256 lanes: four per CU), timed like them: 20 launches per replayed HIP graph."""
+    import ctypes as C
+    dll = microbench_dll()
+    if dll is None:
+        return None
+    stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def fn():
+        rc = dll.fwdmi_mb_empty_launch(grid, block, stream())
+        if rc:
+            raise RuntimeError("empty launch failed: hipError %d" % rc)
+    return time_graph(torch, fn)
+
+
+def hbm_gather(torch, ops, copy_gbs=None, rows=1 << 24, dim=128, n_bags=262144, bag_len=32, steps=20):
+    """The gather rate that is HBM and nothing else: uniform random int32 ids over one fp16 table of
+    2^24 rows x 128 (4 GiB: sixteen times the memory-side cache, 128 times all L2s), 262144 bags of
+    32 ids (8.4 M rows = 2.1 GB of row bytes per launch, 1.7 GB of them distinct), two id sets in
+    turn.  Algorithmic bytes as in the benchmark."""
+    r = np.random.Generator(np.random.PCG64(77))
+    table = torch.empty((rows, dim), dtype=torch.float16, device="cuda")
+    for c0 in range(0, rows, 1 << 21):          # filled in slices: no fp32 copy of the whole table
+        table[c0:c0 + (1 << 21)] = (torch.rand((min(1 << 21, rows - c0), dim), device="cuda") - 0.5) * 0.1
+    sets = []
+    for _ in range(2):
+        ids = torch.from_numpy(r.integers(0, rows, n_bags * bag_len, dtype=np.int64).astype(np.int32)).cuda()
+        sets.append(ids)
+    off = torch.arange(0, n_bags * bag_len, bag_len, dtype=torch.int32, device="cuda")
+    out = torch.empty((n_bags, dim), dtype=torch.float16, device="cuda")
+    n = [0]
+
+    def fn():
+        ops.embedding_bag(table, sets[n[0] & 1], off, "sum", out=out)
+        n[0] += 1
+    _, per = time_events(torch, fn, steps, 5)
+    ms = float(np.mean(per))
+    nbytes = n_bags * bag_len * (dim * 2 + 4) + n_bags * 4 + n_bags * dim * 2
+    res = {"what": "uniform random ids over a 4 GiB fp16 table (2^24 rows x 128): %d bags x %d ids per launch, sum"
+                   % (n_bags, bag_len),
+           "ms": ms, "algorithmic_bytes": nbytes, "algorithmic_GBs": nbytes / (ms * 1e-3) / 1e9,
+           "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           "rows_per_s": n_bags * bag_len / (ms * 1e-3)}
+    if copy_gbs:
+        res["device_copy_GBs"] = copy_gbs
+        res["over_device_copy_rate"] = res["algorithmic_GBs"] / copy_gbs
+    return res
+
+
 def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
     """Tokens/s of the BERT configs and bags/s of config 2.  These launches take ~10 us, less than
     a Python launch costs, so they are timed as HIP-graph replays (GPU time, launch gaps included)."""
@@ -470,10 +551,20 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
         except Exception as e:  # noqa: BLE001
             ex["config2_sum_%s_pytorch_rocm_gpu" % tname] = {"error": repr(e)}
     # these kernels move their algorithmic bytes once (rocprofv3 FETCH_SIZE / WRITE_SIZE agree, see
-    # profiles/): the algorithmic rate over the HBM peak is their roofline position
-    for v in ex.values():
+    # profiles/): the algorithmic rate over the HBM peak is their roofline position.  They are short:
+    # beside it, the same figure with the time of a launch that does nothing taken off.
+    floor = launch_floor_ms(torch)
+    for k, v in ex.items():
         if isinstance(v, dict) and "algorithmic_GBs" in v:
             v["frac_of_hbm_peak"] = v["algorithmic_GBs"] / HBM_PEAK_GBS
+        if floor is not None and isinstance(v, dict) and "ms" in v and "pytorch" not in k and "torch_add" not in k:
+            v["ms_above_launch_floor"] = v["ms"] - floor
+            if "algorithmic_GBs" in v and v["ms"] > floor:
+                v["frac_of_hbm_peak_above_launch_floor"] = v["frac_of_hbm_peak"] * v["ms"] / (v["ms"] - floor)
+    if floor is not None:
+        ex["launch_floor_us"] = floor * 1e3
+        ex["launch_floor_is"] = ("GPU time per launch of a kernel that does nothing (1024 workgroups x 256 lanes), 20 "
+                                 "launches per replayed HIP graph like the figures above")
     return ex
 
 
@@ -563,15 +654,14 @@ def mixed_bag_lengths(torch, ops, workloads, wl, tabs):
 
 
 def replay_times(torch, ops, wl, tabs, idx, off, steps=60):
-    """Times (ms, median of HIP-event durations) of forward_amd/csrc/microbench/replay_gather.hip on the
+    """Times (ms, median of HIP-event durations) of bench_aux/replay_gather.hip on the
     workload's id stream: the rows alone, the rows plus as many stored bytes as the product writes
     (plain / non-temporal stores), and with the stores confined to 4 MiB.  None when the measurement
     aid is not built."""
     import ctypes as C
-    path = os.path.join(ROOT, "forward_amd", "libfwdmi_microbench.so")
-    if not os.path.exists(path):
+    dll = microbench_dll()
+    if dll is None:
         return None
-    dll = C.CDLL(path)
     chunk = 2600                      # ids per workgroup, as the product's runs of 160 bags x 16.3 ids
     it_t, it_s, it_c = [], [], []
     for t in range(len(wl.rows)):
@@ -637,7 +727,7 @@ def replay(torch, ops, workloads, ids_mode):
     del out, batch
     r = replay_times(torch, ops, wl, tabs, idx, off)
     if r is None:
-        raise SystemExit("build the measurement aid first: make -C forward_amd/csrc microbench")
+        raise SystemExit("build the measurement aid first: make -C bench_aux")
     e = r["rows_per_result_row"]
     for label, key in (("gather only (one result row per slot)", "gather_only_ms"),
                        ("gather + a 256 B result row every %d rows, plain stores" % e, "gather_plain_stores_ms"),
@@ -674,7 +764,7 @@ def lru_sim(workloads, capacities=(8192, 12288, 16384, 32768)):
 def main():
     args = parse()
     if args.record_traffic:
-        record_traffic(*args.record_traffic)
+        record_traffic(*args.record_traffic, batches=args.batches)
         return
     if args.lru_sim:
         sys.path.insert(0, ROOT)
@@ -690,6 +780,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU: the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(1)
+    if args.hbm_gather:
+        print(json.dumps(hbm_gather(torch, ops, copy_bandwidth(torch))), flush=True)
+        return
     if args.sweep:
         sweep(torch, ops)
         sweep_layer_norm(torch, ops)
@@ -700,24 +793,33 @@ def main():
 
     t0 = time.time()
     wl = workloads.config4(n_tables=args.tables, n_bags=args.bags)
-    log("ids/offsets generated in %.1fs: %d tables, %d bags each, %d ids, rows %s" %
-        (time.time() - t0, len(wl.rows), wl.n_bags, wl.n_indices(), wl.rows))
+    n_batches = max(1, args.batches)
+    wls = [workloads.config4_fresh_batch(wl, b) for b in range(n_batches)]
+    log("ids/offsets of %d batches generated in %.1fs: %d tables, %d bags each, %d ids in batch 0, rows %s" %
+        (n_batches, time.time() - t0, len(wl.rows), wl.n_bags, wl.n_indices(), wl.rows))
     tabs = device_tables(wl, torch)
-    idx = [torch.from_numpy(i).cuda() for i in wl.indices]
-    off = [torch.from_numpy(o).cuda() for o in wl.offsets]
-    batch = ops.MultiTableBatch(tabs, idx, off)
+    idxs = [[torch.from_numpy(i).cuda() for i in w.indices] for w in wls]
+    offs = [[torch.from_numpy(o).cuda() for o in w.offsets] for w in wls]
+    batches = [ops.MultiTableBatch(tabs, idxs[b], offs[b]) for b in range(n_batches)]
+    idx, off, batch = idxs[0], offs[0], batches[0]
     out = torch.zeros((wl.n_bags, batch.width), dtype=torch.float16, device="cuda")
     torch.cuda.synchronize()
     log("tables resident: %.2f GB, setup %.1fs" % (sum(t.numel() * 2 for t in tabs) / 1e9, time.time() - t0))
 
+    issued = []          # batch number of every step issued so far: step i works on batch i mod B
+
     if args.per_table:
         def step():
+            b = len(issued) % n_batches
+            issued.append(b)
             for t in range(batch.n_tables):
-                ops.embedding_bag(tabs[t], idx[t], off[t], "sum", out=out, out_col=t * wl.dim)
+                ops.embedding_bag(tabs[t], idxs[b][t], offs[b][t], "sum", out=out, out_col=t * wl.dim)
         launches_per_step = batch.n_tables
     else:
         def step():
-            batch.forward(out=out, xcd_table_affinity=not args.no_xcd_affinity)
+            b = len(issued) % n_batches
+            issued.append(b)
+            batches[b].forward(out=out, xcd_table_affinity=not args.no_xcd_affinity)
         launches_per_step = 1
 
     # untimed: brings the engine clock to its steady state, so that a short timed run measures
@@ -726,17 +828,20 @@ def main():
         step()
     torch.cuda.synchronize()
     wall, per = time_events(torch, step, args.steps, args.warmup)
+    timed = issued[-args.steps:]
+    checked_batch = timed[-1]               # `out` now holds this batch's result, written by a timed step
     ms_per_step = wall / args.steps * 1e3
     total_bags = wl.n_bags * len(wl.rows)
-    alg_bytes = wl.algorithmic_bytes(table_itemsize=2, out_itemsize=2, index_itemsize=4)
+    alg_per_batch = [w.algorithmic_bytes(table_itemsize=2, out_itemsize=2, index_itemsize=4) for w in wls]
+    alg_bytes = float(np.mean([alg_per_batch[b] for b in timed]))     # per step, over the steps that were timed
     ev_ms = float(np.mean(per))
     achieved = alg_bytes / (ev_ms * 1e-3) / 1e9
     full = not args.per_table and args.tables == 26 and args.bags == 65536
     comp_bytes, unique_rows = compulsory_bytes(wl)
     # what the 256 vector L1s can return: 64 B per clock and CU at the published peak clock
     l1_peak = torch.cuda.get_device_properties(0).multi_processor_count * 64.0 * MI355X_PEAK_CLOCK_HZ / 1e9
-    traffic = load_traffic() if full else None
-    traffic_bytes = traffic["bag_reduce_config4_bytes_per_launch"] if traffic else None
+    traffic = load_traffic("rotating_batches" if n_batches > 1 else "same_batch") if full else None
+    traffic_bytes = traffic["bytes_per_launch"] if traffic else None
     # Time floor of one launch: the bytes that really cross the L2 boundary (rocprofv3 counters of
     # this launch; the compulsory bytes when no counter figure belongs to this kernel) at the HBM
     # peak, or every algorithmic row byte through the L1s at their return rate, whichever is longer.
@@ -758,36 +863,68 @@ def main():
                    "storage": "fp16 rows and output, fp32 accumulation, int32 ids",
                    "launch": "per-table" if args.per_table else
                    ("fused multi-table" if args.no_xcd_affinity else "fused multi-table, per-XCD table affinity"),
+                   "id_batches": n_batches,
+                   "id_batches_are": ("step i works on batch i mod %d: fresh bag lengths and ids over the same tables, all "
+                                      "resident in HBM before the timed region" % n_batches) if n_batches > 1 else
+                                     "every step replays the same batch",
                    "total_ids": wl.n_indices(), "table_bytes": int(sum(t.numel() * 2 for t in tabs))},
         "roofline": {
-            # `frac` = time floor / kernel time (at most 1); `bound` names the term that sets the floor
-            "bound": "hbm" if floor_hbm_ms >= floor_l1_ms else "l1",
+            "bound": "hbm",
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": floor_ms / ev_ms,
-            "frac_is": "max(hbm-side bytes / 8 TB/s, algorithmic bytes / l1_peak) / kernel time",
+            "frac": achieved / HBM_PEAK_GBS,
+            "frac_is": "algorithmic bytes per launch (every gathered row + its id, offsets, output) / kernel time / HBM "
+                       "peak; above 1 because L1 / L2 serve most row bytes under Zipf ids: not a position under the HBM "
+                       "ceiling, see frac_hbm_side",
+            "frac_algorithmic": achieved / HBM_PEAK_GBS,
+            "frac_algorithmic_is": "the same figure under the name that says what it counts",
             "traffic": traffic_bytes,
-            "hbm_side_bytes_used": hbm_bytes, "hbm_side_bytes_are": "counters" if traffic_bytes else "compulsory",
-            "floor_ms": floor_ms, "floor_hbm_ms": floor_hbm_ms, "floor_l1_ms": floor_l1_ms,
-            # the algorithmic rate against the HBM peak: above 1 when cache hits serve most row bytes,
-            # so it is not a position under the HBM ceiling (kept because the metric names it)
-            "algorithmic_over_hbm_peak": achieved / HBM_PEAK_GBS,
+            "traffic_is": "bytes per launch beyond L2 (rocprofv3 FETCH_SIZE + WRITE_SIZE of this launch in this batch "
+                          "mode, scaled by a 1 GiB copy; memory-side-cache hits included), from profiles/traffic.json",
             "algorithmic_bytes_per_launch": alg_bytes / launches_per_step,
-            "compulsory_bytes_per_step": comp_bytes, "unique_rows": unique_rows,
-            "compulsory_floor_ms": comp_bytes / (HBM_PEAK_GBS * 1e9) * 1e3,
-            "l1_peak_GBs": l1_peak, "l1_frac": achieved / l1_peak,
             "kernel_ms_avg": ev_ms / launches_per_step, "kernel_ms_median": float(np.median(per)),
             "kernel_ms_p10": float(np.percentile(per, 10)),
-            "kernel_ms_p90": float(np.percentile(per, 90)), "launches_per_step": launches_per_step},
+            "kernel_ms_p90": float(np.percentile(per, 90)), "launches_per_step": launches_per_step,
+            # a bounded reading: the longer of "bytes beyond L2 at the HBM peak" and "every row byte through
+            # the L1s at their return rate" over the kernel time
+            "frac_time_floor": floor_ms / ev_ms,
+            "frac_time_floor_is": "max(hbm-side bytes / 8 TB/s, algorithmic bytes / l1_peak) / kernel time",
+            "hbm_side_bytes_used": hbm_bytes, "hbm_side_bytes_are": "counters" if traffic_bytes else "compulsory",
+            "floor_ms": floor_ms, "floor_hbm_ms": floor_hbm_ms, "floor_l1_ms": floor_l1_ms,
+            "compulsory_bytes_batch0": comp_bytes, "unique_rows_batch0": unique_rows,
+            "compulsory_floor_ms": comp_bytes / (HBM_PEAK_GBS * 1e9) * 1e3,
+            "l1_peak_GBs": l1_peak, "l1_frac": achieved / l1_peak},
         "samples_per_s": wl.n_bags / (ms_per_step * 1e-3),
     }
     if traffic_bytes:
         r = result["roofline"]
         # bytes that crossed the L2 boundary (rocprofv3 counters of the same launch) over this run's time
         r["traffic_GBs"] = traffic_bytes / (ev_ms * 1e-3) / 1e9
-        r["hbm_frac"] = r["traffic_GBs"] / HBM_PEAK_GBS
-        r["refetch_ratio"] = traffic["bag_reduce_config4_fetch_bytes"] / float(
-            comp_bytes - len(wl.rows) * wl.n_bags * wl.dim * 2)   # fetched / (distinct rows + ids + offsets)
+        r["frac_hbm_side"] = r["traffic_GBs"] / HBM_PEAK_GBS
+        r["frac_hbm_side_is"] = "traffic / kernel time / HBM peak: what crosses the L2 boundary against the 8 TB/s ceiling"
+        r["refetch_ratio"] = traffic["fetch_bytes"] / float(
+            comp_bytes - len(wl.rows) * wl.n_bags * wl.dim * 2)   # fetched / (distinct rows + ids + offsets), batch 0
         r["traffic_kernel_source_sha256"] = traffic["kernel_source_sha256"]
+    else:
+        result["roofline"]["frac_hbm_side"] = None
+    # the result of the last timed step, kept for the comparison with the oracle below
+    gpu_out_checked = out.cpu().numpy() if not args.no_cpu else None
+
+    if n_batches > 1 and not args.no_extra and not args.per_table:
+        # the figure of a loop that replays one batch: part of its rows is served by the memory-side
+        # cache from the step before, which fresh ids do not get
+        same_step = lambda: batches[0].forward(out=out, xcd_table_affinity=not args.no_xcd_affinity)
+        for _ in range(max(0, args.prewarm)):      # the copy above left the GPU idle: back to the steady clock first
+            same_step()
+        torch.cuda.synchronize()
+        wall1, per1 = time_events(torch, same_step, args.steps, args.warmup)
+        same = {"ms_per_step": wall1 / args.steps * 1e3, "kernel_ms_avg": float(np.mean(per1)),
+                "bags_per_s": total_bags / (wall1 / args.steps),
+                "what": "every step replays batch 0 (the same ids and bag lengths)"}
+        t1 = load_traffic("same_batch") if full else None
+        if t1:
+            same["traffic"] = t1["bytes_per_launch"]
+            same["frac_hbm_side"] = t1["bytes_per_launch"] / (same["kernel_ms_avg"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+        result["same_batch_replay"] = same
 
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
@@ -798,12 +935,18 @@ def main():
         del src, dst
     if not args.no_cpu:
         t1 = time.time()
-        cpu, cpu_out, nb = cpu_baseline(wl, tabs, args.cpu_bags, torch)
-        gpu_out = out[:nb].cpu().numpy()
-        cpu["gpu_matches_oracle_on_sample"] = bool(np.array_equal(gpu_out.view(np.uint16), cpu_out.view(np.uint16)))
-        del gpu_out, cpu_out
+        cpu, cpu_out, nb = cpu_baseline(wls[checked_batch], tabs, args.cpu_bags, torch)
+        cpu["gpu_matches_oracle_on_sample"] = bool(np.array_equal(gpu_out_checked[:nb].view(np.uint16),
+                                                                  cpu_out.view(np.uint16)))
+        cpu["checked"] = "the output of the last timed step (batch %d of %d) against the oracle, bit for bit" % (
+            checked_batch, n_batches)
+        del gpu_out_checked, cpu_out
         result["cpu_baseline"] = cpu
         log("cpu baseline leg %.1fs" % (time.time() - t1))
+    if not args.no_extra:
+        # the side measurements below work on batch 0 and compare with its result
+        batch.forward(out=out, xcd_table_affinity=not args.no_xcd_affinity)
+        torch.cuda.synchronize()
     if not args.no_extra and not args.per_table:
         # the same stage through PyTorch-ROCm's own GPU kernels: 26 embedding_bag launches + cat
         # (a yardstick only: a failure here is recorded, it does not fail the measurement)
@@ -843,9 +986,13 @@ def main():
         except Exception as e:  # noqa: BLE001
             result["mixed_bag_lengths"] = {"error": repr(e)}
     if not args.no_extra:
-        del tabs, batch
+        del tabs, batch, batches, idxs, offs, idx, off
         result["extra"] = extra_measurements(torch, ops, workloads, max(10, args.steps), with_cpu=not args.no_cpu)
         result["extra"]["device_copy_GBs"] = copy_bandwidth(torch)
+        try:
+            result["extra"]["hbm_gather_uniform_4GiB"] = hbm_gather(torch, ops, result["extra"]["device_copy_GBs"])
+        except Exception as e:  # noqa: BLE001
+            result["extra"]["hbm_gather_uniform_4GiB"] = {"error": repr(e)}
     print(json.dumps(result), flush=True)
 
 

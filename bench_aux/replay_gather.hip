@@ -1,4 +1,4 @@
-// Measurement aid, not part of the plugin path: replays the row-id stream of a multi-table bag
+// Measurement aid of bench.py, not part of the plugin path: replays the row-id stream of a multi-table bag
 // workload as the simplest possible gather, to tell what the memory system charges for fetching
 // those rows in that order from what the bag structure (lengths, ordering, per-bag results) adds.
 //
@@ -40,7 +40,9 @@ __device__ __forceinline__ void store_row(Half8 FWDMI_MB_GLOBAL* p, Half8 r, int
   if (mode == 2) {
     U4 x;
     __builtin_memcpy(&x, &r, 16);
-    asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(p), "v"(x) : "memory");
+    // s_nop 1: the wait states a vector write to the data registers of a 128-bit store needs, which the
+    // compiler does not insert behind an asm statement
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(p), "v"(x) : "memory");
   } else {
     *p = r;
   }

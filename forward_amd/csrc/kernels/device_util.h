@@ -51,6 +51,10 @@ __device__ __forceinline__ void gstore(T FWDMI_GLOBAL* p, const Pack<T, N>& r) {
 // staying there as a dirty line that displaces table rows.  For results far larger than the L2s.
 // Written as the instruction itself: a builtin store next to a plain store of the same value (one
 // per branch of a run-time choice) is merged with it by the optimiser and loses the hint.
+// Each store is followed by `s_nop 1`: on this architecture a vector instruction that overwrites the
+// data registers of a store wider than 64 bits needs two wait states behind it, and the compiler, which
+// inserts them for stores it emits itself, does not look inside an asm statement (the registers are
+// dead to it as soon as the statement ends).
 template <typename T, int N>
 __device__ __forceinline__ void gstore_stream(T FWDMI_GLOBAL* p, const Pack<T, N>& r) {
   constexpr int kBytes = (int)sizeof(Pack<T, N>);
@@ -60,14 +64,14 @@ __device__ __forceinline__ void gstore_stream(T FWDMI_GLOBAL* p, const Pack<T, N
   if constexpr (kBytes == 8) {
     U2 x;
     __builtin_memcpy(&x, &r, 8);
-    asm volatile("global_store_dwordx2 %0, %1, off nt" ::"v"(p), "v"(x) : "memory");
+    asm volatile("global_store_dwordx2 %0, %1, off nt\n\ts_nop 1" ::"v"(p), "v"(x) : "memory");
   } else {
     U4 x;
     __builtin_memcpy(&x, &r, 16);
-    asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(p), "v"(x) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(p), "v"(x) : "memory");
     if constexpr (kBytes == 32) {
       __builtin_memcpy(&x, reinterpret_cast<const char*>(&r) + 16, 16);
-      asm volatile("global_store_dwordx4 %0, %1, off offset:16 nt" ::"v"(p), "v"(x) : "memory");
+      asm volatile("global_store_dwordx4 %0, %1, off offset:16 nt\n\ts_nop 1" ::"v"(p), "v"(x) : "memory");
     }
   }
 }

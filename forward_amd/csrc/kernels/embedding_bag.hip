@@ -33,29 +33,14 @@
 #include <type_traits>
 
 #include "../common.h"
+#include "bag_plan.h"
 #include "device_util.h"
 
 namespace fwdmi {
 namespace {
 
-constexpr int kXcds = 8;           // accelerator complex dies; workgroup b is dispatched to XCD b % 8
-constexpr int kWG = 256;           // lanes per workgroup (large batches; small ones use 128 or 64)
-#ifndef FWDMI_BAG_IDX_BYTES
-#define FWDMI_BAG_IDX_BYTES 16384
-#endif
-constexpr int kIdxBytes = FWDMI_BAG_IDX_BYTES;   // LDS bytes of the id window per workgroup (4096 row numbers / 2048 64-bit ids)
-constexpr int kMaxBagsPerWG = 512; // offsets staged in LDS per workgroup (+1)
-constexpr int kLenBuckets = 256;   // bag-length buckets of the in-LDS counting sort
-constexpr int kInlineTables = FWDMI_BAG_INLINE_TABLES;  // table descriptors that travel with the launch as kernel arguments
-constexpr int kMaxVarTables = 64;  // tables of a launch whose runs may differ in size from table to table
 #ifndef FWDMI_BAG_UNROLL
 #define FWDMI_BAG_UNROLL 8
-#endif
-#ifndef FWDMI_BAG_STREAM_BYTES
-#define FWDMI_BAG_STREAM_BYTES (8.0 * 1048576.0)  // results of at least this size are stored with the non-temporal hint
-#endif
-#ifndef FWDMI_BAG_TAIL_RUNS
-#define FWDMI_BAG_TAIL_RUNS(resident) ((resident) / 4)  // measured best on the 26-table configuration (16 .. 384 tried)
 #endif
 #ifndef FWDMI_BAG_WAVES_PER_EU
 #define FWDMI_BAG_WAVES_PER_EU 6  // register budget of 80 VGPRs: measured best on the 26-table configuration
@@ -65,44 +50,6 @@ constexpr int kMaxVarTables = 64;  // tables of a launch whose runs may differ i
 #define FWDMI_BAG_OCCUPANCY \
   __attribute__((amdgpu_waves_per_eu((KIND == kMax || KIND == kSumSq) ? 4 : KIND == kWeighted ? 5 : FWDMI_BAG_WAVES_PER_EU)))
 constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
-
-// kMax also tracks the argmax (needs max_indices); kMaxValue is the plugin's case: values only
-// kSumSq: the sum and the sum of squares of the same rows in one pass (two outputs)
-enum Kind { kPlain = 0, kWeighted = 1, kMax = 2, kSquare = 3, kMaxValue = 4, kSumSq = 5 };
-
-struct BagLaunch {
-  const fwdmi_bag_table* tables;  // device array of descriptors, or nullptr -> `inline_tables`
-  fwdmi_bag_table inline_tables[kInlineTables];  // a single-table launch uses [0]
-  int32_t multi;  // several tables (descriptors in `tables` or inline): weights come with the descriptors
-  const void* psw;  // per-sample weights of the single-table form (a table of a batch carries its own)
-  void* out;
-  void* out2;  // kSumSq: the sums of squares, laid out like `out`
-  void* max_indices;
-  int32_t* oob_flag;
-  int64_t n_bags;
-  int64_t out_stride;
-  int64_t fixed_len;  // >= 0: bag b covers ids [b*fixed_len, (b+1)*fixed_len); < 0: use offsets
-  int32_t dim;
-  int32_t op;
-  int32_t out_f16;
-  int32_t include_last;
-  int32_t log2_g;
-  int32_t n_slices;
-  int32_t bags_per_wg;
-  int32_t wgs_per_table;
-  int32_t vec_store;  // 0: element stores; 1: 16-byte stores; 2: 16-byte stores with the non-temporal hint
-  float one;  // 1.0f
-  int32_t xcd_affinity;      // != 0: XCD x works through work items [xcd_start[x], xcd_start[x+1])
-  int32_t xcd_start[kXcds + 1];
-  int32_t total_wgs;
-  int32_t tail_runs;  // XCD mapping only: the last `tail_runs` runs of every XCD's segment are issued as four workgroups each
-  int32_t idx_cap;    // 32-bit words of the LDS id window: that many row numbers, or half as many 64-bit ids
-  // Multi-table launches whose tables differ in mean bag length: table t's runs hold run_bags[t] bags and
-  // are work items [run_start[t], run_start[t + 1]); bags_per_wg is then the largest of them (it sizes LDS).
-  int32_t var_runs;
-  int32_t run_start[kMaxVarTables + 1];
-  uint16_t run_bags[kMaxVarTables];
-};
 
 // Hands elements first[0 .. n) to put(i, value), the workgroup's lanes sharing the work.  Long
 // ranges come in with 16-byte loads (a load instruction occupies the CU's memory pipeline for the
@@ -145,40 +92,11 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const int wg_lanes = blockDim.x;
 
   const int tid = threadIdx.x;
-  // Each XCD has its own L2.  On request, a multi-table launch undoes the hardware's round-robin
-  // placement (workgroup b runs on XCD b % 8) so that one XCD works through whole tables: a
-  // table's hot rows are then fetched into one L2 instead of all eight.
-  int work = blockIdx.x;
-  int quarter = -1;  // 0..3: this workgroup reduces that quarter of run `work`; -1: the whole run
-  if (L.xcd_affinity) {
-    // A workgroup lives for about an eighth of the launch, so after an XCD has started its last
-    // run its CUs empty out for that long.  The last runs of a segment are therefore cut in four:
-    // their workgroups live a quarter as long and the XCD drains that much faster.
-    const int x = (int)(blockIdx.x % kXcds);
-    const int j = (int)(blockIdx.x / kXcds);
-    const int len = L.xcd_start[x + 1] - L.xcd_start[x];
-    const int tail = min(len, L.tail_runs);
-    const int whole = len - tail;
-    if (j < whole) {
-      work = L.xcd_start[x] + j;
-    } else {
-      const int jj = j - whole;
-      if (jj >= 4 * tail) return;
-      work = L.xcd_start[x] + whole + (jj >> 2);
-      quarter = jj & 3;
-    }
-  }
-  int t, wg, bpw;  // table, run of the table, bags of a run of this table: uniform over the workgroup
-  if (EXT && L.var_runs) {
-    t = 0;
-    while (work >= L.run_start[t + 1]) ++t;  // at most kMaxVarTables steps over kernel arguments
-    wg = work - L.run_start[t];
-    bpw = L.run_bags[t];
-  } else {
-    t = work / L.wgs_per_table;
-    wg = work - t * L.wgs_per_table;
-    bpw = L.bags_per_wg;
-  }
+  // table, run of the table, bags of a run of this table, quarter of the run (-1: the whole run):
+  // uniform over the workgroup
+  BagWork W;
+  if (!bag_decode<EXT>(L, blockIdx.x, &W)) return;
+  const int t = W.table;
   fwdmi_bag_table T;
   if (L.tables) {
     const fwdmi_bag_table FWDMI_GLOBAL* tp = gconst<fwdmi_bag_table>(L.tables) + t;
@@ -199,9 +117,9 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
   const int gl = tid & (G - 1);
   const int slots = wg_lanes >> L.log2_g;
 
-  const int quarter_bags = bpw >> 2;  // the host keeps run sizes multiples of 4 when it cuts runs
-  const int64_t bag0 = (int64_t)wg * bpw + (quarter > 0 ? quarter * quarter_bags : 0);
-  const int nb = (int)min((int64_t)(quarter < 0 ? bpw : quarter_bags), L.n_bags - bag0);
+  int64_t bag0;
+  int nb;
+  bag_run_range(L, W, &bag0, &nb);
   if (nb <= 0) return;  // a quarter beyond the table's last bag (uniform over the workgroup)
   const TI FWDMI_GLOBAL* __restrict__ ids = gconst<TI>(T.input);
   // per-sample weights: the launch's (single table) or the table's own; none = weight 1
@@ -737,6 +655,7 @@ static __device__ __align__(256) unsigned char scratch[kNoAllocMaxTables * sizeo
 // the current device comes from hipGetSymbolAddress, once per device, and is kept here.
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
+std::mutex g_noalloc_issue_mu;  // held while a call enqueues its descriptor writes and its launch
 void* g_scratch_ptr[kMaxDevices] = {};
 
 int scratch_on_current_device(fwdmi_bag_table** out) {
@@ -754,345 +673,92 @@ int scratch_on_current_device(fwdmi_bag_table** out) {
   return FWDMI_OK;
 }
 
-static_assert(sizeof(BagLaunch) <= 4096, "kernel arguments are limited to 4 KiB");
-
-struct BagShape {
-  int grid, block;
-  size_t lds;
-};
-
-// Bytes of the kernel's LDS carve-up.
-size_t bag_lds_bytes(const BagLaunch& L, bool weighted) {
-  size_t b = (size_t)(L.bags_per_wg + 2) * sizeof(int64_t) + (size_t)L.idx_cap * sizeof(uint32_t);
-  if (weighted) b += (size_t)L.idx_cap * sizeof(float);
-  b += (size_t)L.bags_per_wg * (sizeof(int) + sizeof(uint16_t));
-  return (b + 15) & ~(size_t)15;
-}
-
 template <typename TW, typename TI, int VEC, bool EXT>
-int launch_kind_ext(int kind, const BagLaunch& L, const BagShape& sh, hipStream_t stream) {
-  const dim3 grid(sh.grid), block(sh.block);
-  switch (kind) {
+int launch_kind_ext(const BagPlan& P, hipStream_t stream) {
+  const dim3 grid(P.grid), block(P.block);
+  const BagLaunch& L = P.L;
+  switch (P.kind) {
     case kPlain:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kPlain, EXT>), grid, block, sh.lds, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kPlain, EXT>), grid, block, P.lds, stream, L);
       break;
     case kSquare:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSquare, EXT>), grid, block, sh.lds, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSquare, EXT>), grid, block, P.lds, stream, L);
       break;
     case kSumSq:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSumSq, EXT>), grid, block, sh.lds, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kSumSq, EXT>), grid, block, P.lds, stream, L);
       break;
     case kWeighted:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kWeighted, EXT>), grid, block, sh.lds, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kWeighted, EXT>), grid, block, P.lds, stream, L);
       break;
     case kMaxValue:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMaxValue, EXT>), grid, block, sh.lds, stream, L);
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMaxValue, EXT>), grid, block, P.lds, stream, L);
       break;
-    default:
-      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMax, false>), grid, block, sh.lds, stream, L);
+    default:  // argmax: a single table, never the extended form
+      hipLaunchKernelGGL((bag_reduce_kernel<TW, TI, VEC, kMax, false>), grid, block, P.lds, stream, L);
   }
   FWDMI_HIP_CHECK(hipGetLastError());
   return FWDMI_OK;
 }
 
 template <typename TW, typename TI, int VEC>
-int launch_kind(int kind, const BagLaunch& L, const BagShape& sh, hipStream_t stream) {
-  const bool ext = L.var_runs || (L.multi && !L.tables);  // per-table run sizes, or descriptors among the arguments
-  return ext ? launch_kind_ext<TW, TI, VEC, true>(kind, L, sh, stream)
-             : launch_kind_ext<TW, TI, VEC, false>(kind, L, sh, stream);
+int launch_kind(const BagPlan& P, hipStream_t stream) {
+  return P.ext ? launch_kind_ext<TW, TI, VEC, true>(P, stream) : launch_kind_ext<TW, TI, VEC, false>(P, stream);
 }
 
 template <typename TW, typename TI>
-int launch_vec(bool vec, int kind, const BagLaunch& L, const BagShape& sh, hipStream_t stream) {
+int launch_vec(const BagPlan& P, hipStream_t stream) {
   constexpr int kVec = 16 / sizeof(TW);
-  return vec ? launch_kind<TW, TI, kVec>(kind, L, sh, stream)
-             : launch_kind<TW, TI, 1>(kind, L, sh, stream);
+  return P.vec ? launch_kind<TW, TI, kVec>(P, stream) : launch_kind<TW, TI, 1>(P, stream);
 }
 
-int device_cus() {
-  static const int cus = [] {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      return v;
-    return 256;
-  }();
-  return cus;
+// CUs and dies of the current device, asked once per device.  The number of dies is what the
+// runtime reports; a runtime that does not know the attribute leaves the device at one die, and
+// the launch plan then keeps the plain table-major order.
+int device_topology(BagTopology* topo) {
+  static std::mutex mu;
+  static BagTopology known[kMaxDevices] = {};
+  int dev = 0;
+  FWDMI_HIP_CHECK(hipGetDevice(&dev));
+  const bool cached = dev >= 0 && dev < kMaxDevices;
+  std::lock_guard<std::mutex> lock(mu);
+  if (cached && known[dev].cus > 0) {
+    *topo = known[dev];
+    return FWDMI_OK;
+  }
+  BagTopology t{0, 1};
+  FWDMI_HIP_CHECK(hipDeviceGetAttribute(&t.cus, hipDeviceAttributeMultiprocessorCount, dev));
+  FWDMI_REQUIRE(t.cus > 0, "device %d reports %d compute units", dev, t.cus);
+  int xcds = 0;
+  if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, dev) == hipSuccess && xcds > 0)
+    t.xcds = xcds;
+  else
+    (void)hipGetLastError();
+  if (cached) known[dev] = t;
+  *topo = t;
+  return FWDMI_OK;
 }
 
-int next_pow2(int v) {
-  int p = 1;
-  while (p < v) p <<= 1;
-  return p;
-}
-
-// Validates arguments, picks the lane mapping and launches.  `tables_dev` non-null selects the
-// multi-table form with descriptors in device memory, `tables_inline` (host, at most kInlineTables)
-// the one whose descriptors travel as kernel arguments; with neither, `single` is the table.
+// Plans the launch (bag_plan: pure host arithmetic, tested without a GPU) and issues it.
 int bag_dispatch(const fwdmi_bag_table* tables_dev, const fwdmi_bag_table* tables_inline, int n_tables,
                  const fwdmi_bag_table& single,
                  void* output, int64_t n_bags, int64_t fixed_len, int dim, int op, double avg_len,
                  const fwdmi_bag_ext* ext, hipStream_t stream) {
   clear_error();
-  const bool multi = tables_dev || tables_inline;
-  static const fwdmi_bag_ext kDefaultExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr};
-  const fwdmi_bag_ext& x = ext ? *ext : kDefaultExt;
-
-  if (!is_float_dtype(x.table_dtype) || !is_float_dtype(x.out_dtype) || !is_index_dtype(x.index_dtype))
-    return set_error(FWDMI_ERR_UNSUPPORTED, "embedding bag: unsupported dtype (table %d, index %d, out %d)",
-                     x.table_dtype, x.index_dtype, x.out_dtype);
-  if (op != FWDMI_OP_SUM && op != FWDMI_OP_MEAN && op != FWDMI_OP_MAX && op != FWDMI_OP_SQUARE_SUM)
-    return set_error(FWDMI_ERR_UNSUPPORTED, "embedding bag: unknown op %d", op);
-  // dim: a row's byte size and a run's (bag, slice) count stay far inside 32 bits
-  FWDMI_REQUIRE(n_bags >= 0 && dim > 0 && dim <= (1 << 24) && n_tables > 0,
-                "embedding bag: n_bags=%lld dim=%d (1 .. 2^24) n_tables=%d", (long long)n_bags, dim, n_tables);
-  FWDMI_REQUIRE(!(x.per_sample_weights || (multi && (x.flags & FWDMI_BAG_TABLE_WEIGHTS))) || op == FWDMI_OP_SUM,
-                "embedding bag: per_sample_weights needs op SUM (got %d)", op);
-  FWDMI_REQUIRE(!x.max_indices || (op == FWDMI_OP_MAX && !multi),
-                "embedding bag: max_indices needs op MAX on a single table");
-  const int64_t out_stride = x.out_row_stride > 0 ? x.out_row_stride : dim;
-  FWDMI_REQUIRE(out_stride >= dim, "embedding bag: out_row_stride %lld < dim %d", (long long)out_stride, dim);
-  if (n_bags == 0) return FWDMI_OK;
-  FWDMI_REQUIRE(output != nullptr, "embedding bag: null output");
-  if (!multi) {
-    FWDMI_REQUIRE(single.count > 0 && single.data, "embedding bag: empty table");
-    FWDMI_REQUIRE(single.input_size >= 0 && (single.input_size == 0 || single.input),
-                  "embedding bag: null ids");
-    FWDMI_REQUIRE(fixed_len >= 0 || single.input_2, "embedding bag: null offsets");
-    FWDMI_REQUIRE(single.out_col >= 0 && single.out_col + dim <= out_stride, "embedding bag: out_col");
+  // Without a usable device the arguments are still checked first (against a nominal device), so that a
+  // caller learns of a bad argument before it learns of the missing GPU; the device's error stands otherwise.
+  BagTopology topo{256, 8};
+  const int topo_rc = device_topology(&topo);
+  BagPlan P;
+  if (const int rc = bag_plan(tables_dev, tables_inline, n_tables, single, output, n_bags, fixed_len, dim, op, avg_len,
+                              ext, topo, &P))
+    return rc;
+  if (P.empty) {  // no bags: nothing to launch, with or without a device
+    clear_error();
+    return FWDMI_OK;
   }
-
-  const size_t sw = dtype_size(x.table_dtype), so = dtype_size(x.out_dtype);
-  const int vec_w = (int)(16 / sw);
-  // 128-bit row loads need 16-byte row pitch and base; a multi-table launch is checked by its caller.
-  bool vec = (dim % vec_w) == 0;
-  if (!multi) vec = vec && (reinterpret_cast<uintptr_t>(single.data) % 16) == 0;
-  const int VEC = vec ? vec_w : 1;
-
-  BagLaunch L{};
-  L.tables = tables_dev;
-  L.multi = multi;
-  if (tables_inline) {
-    FWDMI_REQUIRE(n_tables <= kInlineTables, "embedding bag: %d tables do not fit the launch's arguments (%d)", n_tables,
-                  kInlineTables);
-    std::copy(tables_inline, tables_inline + n_tables, L.inline_tables);
-  } else {
-    L.inline_tables[0] = single;
-  }
-  L.out = output;
-  L.max_indices = x.max_indices;
-  L.out2 = x.square_sum_out;
-  L.oob_flag = x.oob_flag;
-  L.n_bags = n_bags;
-  L.out_stride = out_stride;
-  L.fixed_len = fixed_len;
-  L.one = 1.0f;
-  L.dim = dim;
-  L.op = op;
-  L.out_f16 = x.out_dtype == FWDMI_F16;
-  L.include_last = x.include_last_offset != 0;
-  const int lanes = std::min(64, next_pow2((dim + VEC - 1) / VEC));
-  L.log2_g = __builtin_ctz(lanes);
-  L.n_slices = (dim + lanes * VEC - 1) / (lanes * VEC);
-  if (avg_len < 1.0) avg_len = 1.0;
-  // Run length: as many bags as keep the run's ids inside the LDS window, but no more than leaves
-  // the chip with ~4 workgroups per CU; small batches also shrink the workgroup (down to one
-  // wavefront) so that every CU gets work, but not below one slot per bag of the run: a slot
-  // that reduces two bags one after the other doubles the launch's critical path.
-  // The id window is sized for 32-bit row numbers unless a single table is known to be too large
-  // for them (more than 2^24 rows or 4 GiB): then it holds the launch's 64-bit ids.  (A multi-table
-  // launch cannot see its tables' sizes here; a run of such a table that does not fit the window
-  // reads its ids from global memory.)
-  const bool i64_ids = x.index_dtype == FWDMI_I64;
-  const bool wide_ids = i64_ids && !multi &&
-                        (single.count > (1 << 24) || (uint64_t)single.count * dim * sw > ((uint64_t)1 << 32));
-  const int max_cap = kIdxBytes / (wide_ids ? 8 : 4);
-  const int64_t total_bags = n_bags * n_tables;
-  const int64_t target_wgs = (int64_t)device_cus() * 4;
-  int64_t want_bags = std::max<int64_t>(1, total_bags / target_wgs);
-  const int64_t fit_bags = std::max<int64_t>(1, (int64_t)(max_cap / 2.0 / avg_len));
-  want_bags = std::min<int64_t>(std::min(want_bags, fit_bags), kMaxBagsPerWG);
-  int block = kWG;
-  while (block > 64 && block / 2 >= lanes && (int64_t)(block / 2 / lanes) >= want_bags * L.n_slices) block /= 2;
-  const int slots = block / lanes;
-  // Bags of a run and words of its id window for bags of `avg` ids on average.
-  const bool weighted_launch = x.per_sample_weights || (multi && (x.flags & FWDMI_BAG_TABLE_WEIGHTS));
-  auto size_run = [&](double avg, int64_t want, int* bags, int* cap) {
-    // a whole number of rounds over the slots
-    const int64_t units = std::max<int64_t>(slots, want * L.n_slices / slots * slots);
-    *bags = (int)std::max<int64_t>(1, std::min<int64_t>(kMaxBagsPerWG, units / L.n_slices));
-    *cap = std::min(max_cap, std::max(64, next_pow2((int)std::min<double>(max_cap, avg * *bags * 2.0)))) * (wide_ids ? 2 : 1);
-    // With per-sample weights every window slot also holds a weight, and at twice the expected ids the
-    // two windows (35 KiB for a run of 112 bags) leave a CU four workgroups.  The expected ids plus 5.5
-    // times the spread of a sum of `bags` lengths whose deviation equals their mean keeps all
-    // but one run in ten thousand staged (a run that reads its ids unstaged takes several times as
-    // long: at 4 spreads, 0.25 % of the runs unstaged, the launch below measures 0.466 ms); measured on
-    // the 26-table configuration: 0.490 -> 0.440 ms together with the register budget above.
-    if (weighted_launch) {
-      const double ids = avg * (*bags + 5.5 * std::sqrt((double)*bags));
-      const int tight = ((int)std::min<double>(max_cap, std::max(64.0, ids)) + 63) / 64 * 64 * (wide_ids ? 2 : 1);
-      *cap = std::min(*cap, tight);
-    }
-  };
-  size_run(avg_len, want_bags, &L.bags_per_wg, &L.idx_cap);
-  // Tables whose mean bag lengths differ (one-hot features beside multi-hot ones) get runs of their
-  // own size: sized from the launch's mean, the runs of a long-bag table overflow the id window and
-  // those of a one-hot table hold a few ids each.  Measured on 13 one-hot + 13 long-bag tables
-  // (28.6 M ids): 0.562 ms with one run size.
-  int run_bags[kMaxVarTables];
-  bool var_runs = false;
-  if (multi && x.table_avg_len && n_tables > 1 && n_tables <= kMaxVarTables) {
-    const int64_t want_all = std::min<int64_t>(std::max<int64_t>(1, total_bags / target_wgs), kMaxBagsPerWG);
-    int lo = INT_MAX, hi = 0, cap_max = 0;
-    for (int t = 0; t < n_tables; ++t) {
-      const double a = (double)x.table_avg_len[t];
-      FWDMI_REQUIRE(a >= 0.0 && a < 1e30, "embedding bag: table_avg_len must be finite and not negative");
-      const double avg_t = std::max(1.0, a);
-      const int64_t fit_t = std::max<int64_t>(1, (int64_t)(max_cap / 2.0 / avg_t));
-      int cap_t = 0;
-      size_run(avg_t, std::min(want_all, fit_t), &run_bags[t], &cap_t);
-      lo = std::min(lo, run_bags[t]);
-      hi = std::max(hi, run_bags[t]);
-      cap_max = std::max(cap_max, cap_t);
-    }
-    if (2 * hi >= 3 * lo) {  // otherwise one size serves all tables
-      var_runs = true;
-      L.bags_per_wg = hi;
-      L.idx_cap = cap_max;
-    }
-  }
-  const int64_t wgs = (n_bags + L.bags_per_wg - 1) / L.bags_per_wg;
-  FWDMI_REQUIRE(wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
-  L.wgs_per_table = (int)wgs;
-  int64_t total_runs = wgs * n_tables;
-  L.var_runs = 0;
-  if (var_runs) {
-    total_runs = 0;
-    for (int t = 0; t < n_tables; ++t) {
-      L.run_start[t] = (int32_t)total_runs;
-      L.run_bags[t] = (uint16_t)run_bags[t];
-      total_runs += (n_bags + run_bags[t] - 1) / run_bags[t];
-      FWDMI_REQUIRE(total_runs < (int64_t)1 << 31, "embedding bag: grid too large");
-    }
-    L.run_start[n_tables] = (int32_t)total_runs;
-    L.var_runs = 1;
-  }
-  const size_t store_align = std::min<size_t>(16, VEC * so);
-  L.vec_store = VEC > 1 && (reinterpret_cast<uintptr_t>(output) % store_align) == 0 &&
-                (reinterpret_cast<uintptr_t>(x.square_sum_out) % store_align) == 0 &&
-                ((out_stride * so) % store_align) == 0 &&
-                (multi || (single.out_col * so) % store_align == 0);
-
-  // A result of several MiB does not survive in the 4 MiB L2 of the XCD that wrote it until somebody
-  // reads it (and a reader on another XCD would not find it there anyway); written with the
-  // non-temporal hint it does not displace table rows on its way out.  Measured: 2.8 % off the
-  // 26-table launch (19 % when every row hits in cache), 3.8 % off 26 single-table launches of
-  // 16 MiB results each; a reader of a 16 MiB result right behind the launch costs 2 % more.
-  if (L.vec_store && (double)n_bags * n_tables * dim * so >= FWDMI_BAG_STREAM_BYTES) L.vec_store = 2;
-
-  const bool weighted = weighted_launch;
-  FWDMI_REQUIRE(!x.square_sum_out || (op == FWDMI_OP_SUM && !weighted),
-                "embedding bag: square_sum_out needs op SUM without per-sample weights");
-  const int kind = op == FWDMI_OP_MAX      ? (x.max_indices ? kMax : kMaxValue)
-                   : op == FWDMI_OP_SQUARE_SUM ? kSquare
-                   : weighted                  ? kWeighted
-                   : x.square_sum_out          ? kSumSq
-                                               : kPlain;
-  L.psw = x.per_sample_weights;
-  int grid = (int)total_runs;
-  L.total_wgs = grid;
-  L.xcd_affinity = 0;
-  if (multi && n_tables > 1 && (x.flags & FWDMI_BAG_XCD_TABLE_AFFINITY)) {
-    // Cut the table-major work list into eight contiguous segments of equal estimated cost
-    // (equal length when the caller gives no per-table cost).
-    L.xcd_affinity = 1;
-    // A bag costs its rows plus a constant (result store, bookkeeping) worth kBagRows rows: fixed-length
-    // launches of 1 .. 64 rows per bag fit rows / 36.6 TB/s + result bytes / 3.7 TB/s, and one-hot
-    // tables beside tables of 33 ids per bag measure 1 : 4.1 per bag.  With every table's mean bag
-    // length known the caller's per-bag cost is scaled by it; without, all tables count as equally long.
-    constexpr double kBagRows = 9.6;
-    auto cost_of = [&](int u) {
-      double c = x.table_cost ? (double)x.table_cost[u] : 1.0;
-      if (x.table_avg_len) c *= (std::max(0.0, (double)x.table_avg_len[u]) + kBagRows) / (avg_len + kBagRows);
-      return c;
-    };
-    double total = 0.0;
-    for (int t = 0; t < n_tables; ++t) {
-      const double c = cost_of(t);
-      FWDMI_REQUIRE(c > 0.0 && c < 1e30, "embedding bag: table_cost must be positive and finite");
-      const double a = x.table_avg_len ? (double)x.table_avg_len[t] : 0.0;
-      FWDMI_REQUIRE(a >= 0.0 && a < 1e30, "embedding bag: table_avg_len must be finite and not negative");
-      total += cost_of(t) * (double)wgs;
-    }
-    int t = 0;
-    double before = 0.0;  // cost of the tables before t
-    int longest = 0;
-    L.xcd_start[0] = 0;
-    if (var_runs) {
-      // the same cut with runs whose size differs from table to table: a table's cost is its bags' cost
-      double all = 0.0;
-      for (int u = 0; u < n_tables; ++u) all += cost_of(u) * (double)n_bags;
-      for (int k = 1; k <= kXcds; ++k) {
-        int cut = grid;
-        if (k < kXcds) {
-          const double target = all * k / kXcds;
-          double c = cost_of(t);
-          while (t < n_tables - 1 && before + c * (double)n_bags <= target) {
-            before += c * (double)n_bags;
-            ++t;
-            c = cost_of(t);
-          }
-          const int64_t runs_t = L.run_start[t + 1] - L.run_start[t];
-          const int64_t within =
-              std::min<int64_t>(runs_t, std::max<int64_t>(0, (int64_t)((target - before) / (c * run_bags[t]) + 0.5)));
-          cut = (int)std::max<int64_t>(L.xcd_start[k - 1], (int64_t)L.run_start[t] + within);
-        }
-        L.xcd_start[k] = cut;
-        longest = std::max(longest, cut - L.xcd_start[k - 1]);
-      }
-    } else {
-      for (int k = 1; k <= kXcds; ++k) {
-        int cut = grid;
-        if (k < kXcds) {
-          const double target = total * k / kXcds;
-          double c = cost_of(t);
-          while (t < n_tables - 1 && before + c * (double)wgs <= target) {
-            before += c * (double)wgs;
-            ++t;
-            c = cost_of(t);
-          }
-          const int64_t within = std::min<int64_t>(wgs, std::max<int64_t>(0, (int64_t)((target - before) / c + 0.5)));
-          cut = (int)std::max<int64_t>(L.xcd_start[k - 1], (int64_t)t * wgs + within);
-        }
-        L.xcd_start[k] = cut;
-        longest = std::max(longest, cut - L.xcd_start[k - 1]);
-      }
-    }
-    // Runs cut in four at the end of every segment (see the kernel): as many as a quarter of what an XCD holds
-    // at once, and only in launches that fill the chip several times over.
-    const int resident = device_cus() / kXcds * 6;  // workgroups of 256 lanes an XCD holds at the 6-per-CU occupancy
-    L.tail_runs = 0;
-    bool can_cut = block == kWG && L.bags_per_wg % 4 == 0 && L.bags_per_wg / 4 >= slots;
-    for (int u = 0; var_runs && u < n_tables; ++u) can_cut = can_cut && run_bags[u] % 4 == 0 && run_bags[u] / 4 >= slots;
-    if (can_cut && longest >= 4 * resident) L.tail_runs = FWDMI_BAG_TAIL_RUNS(resident);
-#ifdef FWDMI_EXP_ENV
-    if (const char* e = getenv("FWDMI_EXP_TAIL_RUNS")) L.tail_runs = atoi(e);
-#endif
-    int most = 0;  // workgroups of the XCD with the most
-    for (int k = 0; k < kXcds; ++k) {
-      const int len = L.xcd_start[k + 1] - L.xcd_start[k];
-      most = std::max(most, len + 3 * std::min(len, L.tail_runs));
-    }
-    FWDMI_REQUIRE((int64_t)most * kXcds < (int64_t)1 << 31, "embedding bag: grid too large");
-    grid = most * kXcds;
-  }
-  const bool f16 = x.table_dtype == FWDMI_F16, i64 = x.index_dtype == FWDMI_I64;
-  const BagShape sh{grid, block, bag_lds_bytes(L, kind == kWeighted)};
-  if (f16)
-    return i64 ? launch_vec<_Float16, int64_t>(vec, kind, L, sh, stream)
-               : launch_vec<_Float16, int32_t>(vec, kind, L, sh, stream);
-  return i64 ? launch_vec<float, int64_t>(vec, kind, L, sh, stream)
-             : launch_vec<float, int32_t>(vec, kind, L, sh, stream);
+  if (topo_rc) return topo_rc;
+  if (P.f16) return P.i64 ? launch_vec<_Float16, int64_t>(P, stream) : launch_vec<_Float16, int32_t>(P, stream);
+  return P.i64 ? launch_vec<float, int64_t>(P, stream) : launch_vec<float, int32_t>(P, stream);
 }
 
 }  // namespace
@@ -1192,9 +858,10 @@ int check_host_tables(const char* what, const fwdmi_bag_table* tables_host, int3
 // Every table's own mean bag length, from host descriptors, unless the caller gave them.
 void fill_avg_len(fwdmi_bag_ext* x, float* avg_len_t, const fwdmi_bag_table* tables_host, int32_t n_tables,
                   int64_t n_bags) {
-  if (x->table_avg_len || n_tables > fwdmi::kMaxVarTables || n_bags <= 0) return;
+  if ((x->flags & FWDMI_BAG_TABLE_AVG_LEN) || n_tables > fwdmi::kMaxVarTables || n_bags <= 0) return;
   for (int32_t t = 0; t < n_tables; ++t) avg_len_t[t] = (float)((double)tables_host[t].input_size / (double)n_bags);
   x->table_avg_len = avg_len_t;
+  x->flags |= FWDMI_BAG_TABLE_AVG_LEN;
 }
 
 const fwdmi_bag_ext kPlainExt = {FWDMI_F32, FWDMI_I32, FWDMI_F32, 0, nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr};
@@ -1243,16 +910,23 @@ int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_
                             "(FWDMI_BAG_TABLE_WEIGHTS), not into ext->per_sample_weights");
   // the descriptors are host memory here, so what the device form leaves to its caller is checked
   if (const int rc = check_host_tables(kWhat, tables_host, n_tables, dim, ext)) return rc;
-  fwdmi_bag_table* dev_tables = nullptr;
-  if (const int rc = fwdmi::scratch_on_current_device(&dev_tables)) return rc;
-  // stream order keeps a call's descriptors intact until its launch has read them, as long as
-  // every call on this GPU uses the same stream (or the caller orders them)
-  if (const int rc = fwdmi_bag_tables_fill(tables_host, n_tables, dev_tables, stream)) return rc;
   fwdmi_bag_table none{};
   // the descriptors are on the host here: every table's own mean bag length comes with them
   fwdmi_bag_ext with_len = ext ? *ext : kPlainExt;
   float avg_len_t[fwdmi::kMaxVarTables];
   fill_avg_len(&with_len, avg_len_t, tables_host, n_tables, n_bags);
+  // Few enough tables travel with the launch as kernel arguments: nothing is shared between calls then.
+  if (n_tables <= fwdmi::kInlineTables)
+    return fwdmi::bag_dispatch(nullptr, tables_host, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len,
+                               &with_len, static_cast<hipStream_t>(stream));
+  fwdmi_bag_table* dev_tables = nullptr;
+  if (const int rc = fwdmi::scratch_on_current_device(&dev_tables)) return rc;
+  // The descriptor writes and the launch that reads them are enqueued under one lock, so that two host
+  // threads issuing on the same stream cannot interleave them; stream order then keeps a call's
+  // descriptors intact until its launch has read them.  Calls on different streams of one GPU still
+  // race unless the caller orders them.
+  std::lock_guard<std::mutex> lock(fwdmi::g_noalloc_issue_mu);
+  if (const int rc = fwdmi_bag_tables_fill(tables_host, n_tables, dev_tables, stream)) return rc;
   return fwdmi::bag_dispatch(dev_tables, nullptr, n_tables, none, output, n_bags, -1, dim, op_type, avg_bag_len, &with_len,
                              static_cast<hipStream_t>(stream));
 }

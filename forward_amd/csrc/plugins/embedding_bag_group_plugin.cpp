@@ -222,6 +222,7 @@ int EmbeddingBagGroupPlugin::enqueue(const PluginTensorDesc* inputDesc, const Pl
   if (T <= kMaxLenHints) {
     for (int t = 0; t < T; ++t) avg_len_t[t] /= (float)n_bags;
     x.table_avg_len = avg_len_t;
+    x.flags |= FWDMI_BAG_TABLE_AVG_LEN;
   }
   const double avg_len = (double)total_ids / ((double)n_bags * T);
   if (T <= FWDMI_BAG_INLINE_TABLES)  // `chunk` holds them all: the descriptors are kernel arguments of the one launch

@@ -25,6 +25,7 @@ FORMAT_LINEAR = 0
 OP_SUM, OP_MEAN, OP_MAX, OP_SQUARE_SUM, OP_GATHER = 0, 1, 2, 3, 999
 BAG_XCD_TABLE_AFFINITY = 1
 BAG_TABLE_WEIGHTS = 2
+BAG_TABLE_AVG_LEN = 4
 BAG_INLINE_TABLES = 40        # FWDMI_BAG_INLINE_TABLES
 
 

@@ -54,7 +54,7 @@ def _ext(table, indices, out_dtype, include_last_offset=False, psw=None, max_ind
     x.max_indices = max_indices.data_ptr() if max_indices is not None else None
     x.out_row_stride = int(out_row_stride)
     x.oob_flag = oob_flag.data_ptr() if oob_flag is not None else None
-    x.flags = flags
+    x.flags = flags | (lib.BAG_TABLE_AVG_LEN if table_avg_len is not None else 0)
     x.table_cost = table_cost.ctypes.data if table_cost is not None else None
     x.square_sum_out = square_sum_out.data_ptr() if square_sum_out is not None else None
     x.table_avg_len = table_avg_len.ctypes.data if table_avg_len is not None else None

@@ -194,6 +194,17 @@ class MultiTableWorkload:
         return ((x - np.float32(0.5)) * np.float32(0.1)).astype(dtype)
 
 
+def _config4_ids(rng, rows, n_bags, len_cdf, max_len, len_s, idx_s):
+    """One batch of the sparse stage: per table, Zipf bag lengths and Zipf ids scattered over the rows."""
+    indices, offsets = [], []
+    for r in rows:
+        lengths = zipf_ranks(rng, max_len, len_s, n_bags, len_cdf).astype(np.int64) + 1
+        n = int(lengths.sum())
+        indices.append(scatter_ranks(zipf_ranks(rng, r, idx_s, n), r).astype(np.int32))
+        offsets.append(offsets_from_lengths(lengths, np.int32))
+    return indices, offsets
+
+
 def config4(variant=0, n_tables=26, n_bags=65536, dim=128, min_rows=1e3, max_rows=1e7,
             len_s=1.1, idx_s=1.1, max_len=100):
     """26 tables, rows log-uniform in [1e3, 1e7]; bag lengths truncated Zipf(1.1) on 1..100
@@ -202,12 +213,18 @@ def config4(variant=0, n_tables=26, n_bags=65536, dim=128, min_rows=1e3, max_row
     lo, hi = np.log10(min_rows), np.log10(max_rows)
     rows = [int(round(10 ** u)) for u in rng.uniform(lo, hi, size=n_tables)]
     w = MultiTableWorkload(rows, dim, n_bags)
-    len_cdf = zipf_cdf(max_len, len_s)
-    for t in range(n_tables):
-        lengths = zipf_ranks(rng, max_len, len_s, n_bags, len_cdf).astype(np.int64) + 1
-        n = int(lengths.sum())
-        idx = scatter_ranks(zipf_ranks(rng, rows[t], idx_s, n), rows[t]).astype(np.int32)
-        w.indices.append(idx)
-        w.offsets.append(offsets_from_lengths(lengths, np.int32))
-        w.table_seeds.append(1000 * 4 + 100 * (variant + 1) + t)
+    w.indices, w.offsets = _config4_ids(rng, rows, n_bags, zipf_cdf(max_len, len_s), max_len, len_s, idx_s)
+    w.table_seeds = [1000 * 4 + 100 * (variant + 1) + t for t in range(n_tables)]
     return w
+
+
+def config4_fresh_batch(w, batch, len_s=1.1, idx_s=1.1, max_len=100):
+    """Another batch of samples for the tables of ``w`` (same rows, same table seeds): new bag
+    lengths and ids from the same distributions, seeded by ``batch`` (>= 1; batch 0 is ``w`` itself).
+    A serving loop never sees the same ids twice: the benchmark cycles through several of these."""
+    if batch == 0:
+        return w
+    rng = rng_for(4, 500 + int(batch))
+    b = MultiTableWorkload(list(w.rows), w.dim, w.n_bags, table_seeds=list(w.table_seeds))
+    b.indices, b.offsets = _config4_ids(rng, w.rows, w.n_bags, zipf_cdf(max_len, len_s), max_len, len_s, idx_s)
+    return b

@@ -95,13 +95,16 @@ typedef struct fwdmi_bag_ext {
                                   bag: the two reductions a factorisation-machine term needs
                                   (the reference builds them as two plugins over two copies of
                                   the table, source/fwd_tf/tf_cvt/tf_desc_creators/tf_embedding_bag_creator.h:43-95) */
-  const float* table_avg_len;  /* HOST array [n_tables] or NULL: mean ids per bag of each table of a
-                                  multi-table launch.  With it, a table's share of the XCD segments
-                                  (FWDMI_BAG_XCD_TABLE_AFFINITY) follows its bags' length as well as
-                                  table_cost, and in launches of at most 64 tables those whose means
-                                  differ by half or more get runs of their own size; without it every
-                                  table counts as avg_bag_len long.  A sizing hint only: results do
-                                  not depend on it */
+  const float* table_avg_len;  /* read only with FWDMI_BAG_TABLE_AVG_LEN in `flags`.  HOST array [n_tables]
+                                  or NULL: mean ids per bag of each table of a multi-table launch.  With
+                                  it, a table's share of the XCD segments (FWDMI_BAG_XCD_TABLE_AFFINITY)
+                                  follows its bags' length as well as table_cost, and in launches of at
+                                  most 64 tables those whose means differ by half or more get runs of
+                                  their own size; without it every table counts as avg_bag_len long.  A
+                                  sizing hint only: results do not depend on it */
+  /* Layout of library version 0.2 (fwdmi_version()).  Members added after it are announced by a
+   * bit in `flags` and read only when that bit is set, so a caller built against this layout
+   * keeps working with later libraries. */
 } fwdmi_bag_ext;
 
 /* Multi-table launches only: renumber workgroups so that each of the 8 XCDs (one L2 each)
@@ -114,6 +117,8 @@ typedef struct fwdmi_bag_ext {
  * (per-sample weights in the table's type, one per id); a table whose pointer is NULL uses
  * weight 1 for all of its ids. */
 #define FWDMI_BAG_TABLE_WEIGHTS 2
+/* ext->table_avg_len is present and may be read (see there). */
+#define FWDMI_BAG_TABLE_AVG_LEN 4
 
 /*
  * Variable-length bags: bag b = input[input_2[b] .. input_2[b+1]), last bag ends at input_size.
@@ -185,7 +190,8 @@ int fwdmi_embedding_bag_multi(const fwdmi_bag_table* tables_dev, int32_t n_table
  * More tables are written to `tables_dev` (a device array of n_tables descriptors, required then) by
  * fwdmi_bag_tables_fill on the same stream first.  The descriptors are checked on the host (data /
  * ids / offsets present, column block inside the output row, 16-byte alignment where rows are read as
- * slices) and every table's mean bag length is taken from them unless ext->table_avg_len is given.
+ * slices) and, for at most 64 tables, every table's mean bag length is taken from them unless
+ * ext->table_avg_len is given (more tables run with avg_bag_len for all of them).
  * Results equal those of fwdmi_embedding_bag_multi bit for bit.
  */
 #define FWDMI_BAG_INLINE_TABLES 40
@@ -201,10 +207,13 @@ int fwdmi_embedding_bag_multi_host(const fwdmi_bag_table* tables_host, int32_t n
  * launches exactly what fwdmi_embedding_bag_multi launches, so results are bit-identical.
  * It calls no hipMalloc / hipFree or any other allocating routine; inputs and outputs are the
  * caller's.  Limits: at most 1024 tables per call (more is FWDMI_ERR_BAD_ARG; the buffer holds
- * 64 KiB per GPU for the life of the process).  Every call on one GPU shares that GPU's buffer:
- * calls on the same stream are ordered by it; calls that overlap on one GPU (different streams
- * without an ordering between them) race and must not be made.  The first call on a device looks
- * the buffer's address up (hipGetSymbolAddress); make that call outside a graph capture.
+ * 64 KiB per GPU for the life of the process).  Calls of at most FWDMI_BAG_INLINE_TABLES tables
+ * carry their descriptors among the launch's own arguments and share nothing.  Larger calls on
+ * one GPU share that GPU's buffer: a call's descriptor writes and its launch are enqueued under
+ * one lock, so calls on the same stream, from any number of host threads, are ordered by the
+ * stream; calls that overlap on one GPU (different streams without an ordering between them)
+ * race and must not be made.  The first such call on a device looks the buffer's address up
+ * (hipGetSymbolAddress); make that call outside a graph capture.
  */
 int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_t n_tables, int64_t n_bags,
                                       void* output, int32_t dim, int32_t op_type, double avg_bag_len,

@@ -2,7 +2,9 @@
 device memory (its descriptor buffer is part of the library's code object).  Called through the
 C ABI and compared bit for bit with fwdmi_embedding_bag_multi on the same inputs, on two calls in
 a row, the second with a smaller input (fewer tables, fewer bags), so that what the first call
-left in the shared buffer must not leak into the second."""
+left in the shared buffer must not leak into the second.  Calls of more than
+FWDMI_BAG_INLINE_TABLES tables go through that buffer; smaller ones carry their descriptors among
+the launch's arguments: both sizes are covered."""
 import ctypes as C
 
 import numpy as np
@@ -53,11 +55,18 @@ def launch_both(tables, ids, offs, dim, op, flags):
 
 
 @pytest.mark.parametrize("tdt,idt", [(np.float16, np.int32), (np.float32, np.int64)])
-def test_no_alloc_entry_point_equals_the_allocating_form_twice_in_a_row(oracle, tdt, idt):
+@pytest.mark.parametrize("through_buffer", [True, False])
+def test_no_alloc_entry_point_equals_the_allocating_form_twice_in_a_row(oracle, tdt, idt, through_buffer):
     rng = np.random.Generator(np.random.PCG64(2024))
     dim = 128 if tdt == np.float16 else 64
-    first = make_batch(rng, [4000, 17, 90000, 512, 30000, 7, 1200, 65000, 300], 3000, dim, tdt, idt, 24)
-    second = make_batch(rng, [900, 20000, 5], 257, dim, tdt, idt, 9)        # smaller: 3 tables, 257 bags
+    rows1 = [4000, 17, 90000, 512, 30000, 7, 1200, 65000, 300]
+    rows2 = [900, 20000, 5]
+    if through_buffer:          # more tables than travel with a launch: the built-in descriptor buffer is used
+        rows1 = rows1 + [int(v) for v in rng.integers(3, 5000, lib.BAG_INLINE_TABLES + 8 - len(rows1))]
+        rows2 = rows2 + [int(v) for v in rng.integers(3, 5000, lib.BAG_INLINE_TABLES + 2 - len(rows2))]
+        assert len(rows2) > lib.BAG_INLINE_TABLES and len(rows2) < len(rows1)
+    first = make_batch(rng, rows1, 3000, dim, tdt, idt, 24)
+    second = make_batch(rng, rows2, 257, dim, tdt, idt, 9)        # smaller: fewer tables, 257 bags
     for call, (tables, ids, offs) in enumerate((first, second)):
         for op in (ops.MODES["sum"], ops.MODES["max"]):
             want, got = launch_both(tables, ids, offs, dim, op, lib.BAG_XCD_TABLE_AFFINITY if call == 0 else 0)
@@ -65,6 +74,48 @@ def test_no_alloc_entry_point_equals_the_allocating_form_twice_in_a_row(oracle, 
             for t, tab in enumerate(tables):                                  # and both against the oracle
                 ref, _, _ = oracle.embedding_bag(tab, ids[t], offs[t], op)
                 assert_bits_equal(got[:, t * dim:(t + 1) * dim], ref, "call %d table %d against the oracle" % (call, t))
+
+
+@pytest.mark.parametrize("affinity", [False, True])
+def test_many_tables_of_very_different_bag_lengths_with_descriptors_in_device_memory(oracle, affinity):
+    """48 tables, one-hot ones alternating with long-bag ones: more tables than travel with a launch, few
+    enough for runs sized per table, so the kernel takes per-table run sizes while it reads its descriptors
+    from device memory.  Through fwdmi_embedding_bag_multi_host with a caller's device array and through the
+    no-allocation entry point, with and without the per-XCD mapping; whole output against the oracle."""
+    rng = np.random.Generator(np.random.PCG64(48))
+    n_tables, dim, n_bags = 48, 64, 6000
+    rows = [int(v) for v in rng.integers(50, 30000, n_tables)]
+    tables = [(rng.standard_normal((r, dim)) * 0.3).astype(np.float16) for r in rows]
+    ids, offs = [], []
+    for t, r in enumerate(rows):
+        lengths = np.ones(n_bags, np.int64) if t % 2 == 0 else rng.poisson(45, n_bags)
+        if t == 7:
+            lengths[100:104] = 5000            # bags longer than the id window
+            lengths[3::50] = 0
+        offs.append(np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(np.int32))
+        ids.append(rng.integers(0, r, int(lengths.sum())).astype(np.int32))
+    want = np.zeros((n_bags, n_tables * dim), np.float16)
+    for t in range(n_tables):
+        oracle.embedding_bag(tables[t], ids[t], offs[t], oracle.OP_SUM, out=want, out_col=dim * t)
+    d_tab, d_ids, d_off = [dev(t) for t in tables], [dev(i) for i in ids], [dev(o) for o in offs]
+    desc = descriptors(d_tab, d_ids, d_off, dim)
+    avg = float(sum(i.size for i in ids)) / (n_tables * n_bags)
+    s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    flags = lib.BAG_XCD_TABLE_AFFINITY if affinity else 0
+    d_desc = torch.empty(n_tables * 64, dtype=torch.uint8, device="cuda")
+    for name in ("host descriptors + device array", "no allocation"):
+        out = torch.full((n_bags, n_tables * dim), -3.0, dtype=torch.float16, device="cuda")
+        x = ops._ext(d_tab[0], d_ids[0], torch.float16, out_row_stride=n_tables * dim, flags=flags)
+        if name == "no allocation":
+            rc = lib.dll.fwdmi_embedding_bag_multi_noalloc(C.c_void_p(desc.ctypes.data), n_tables, n_bags,
+                                                           C.c_void_p(out.data_ptr()), dim, 0, avg, C.byref(x), s)
+        else:
+            rc = lib.dll.fwdmi_embedding_bag_multi_host(C.c_void_p(desc.ctypes.data), n_tables,
+                                                        C.c_void_p(d_desc.data_ptr()), n_bags,
+                                                        C.c_void_p(out.data_ptr()), dim, 0, avg, C.byref(x), s)
+        lib.check(rc)
+        torch.cuda.synchronize()
+        assert_bits_equal(host(out), want, "%s, affinity %s" % (name, affinity))
 
 
 def test_no_alloc_entry_point_limits_and_argument_errors():
@@ -123,12 +174,13 @@ def test_no_alloc_entry_point_on_config4_at_full_size():
     assert torch.equal(got, want)
 
 
-def test_no_alloc_entry_point_under_graph_capture(oracle):
+@pytest.mark.parametrize("n_tables", [3, lib.BAG_INLINE_TABLES + 4])
+def test_no_alloc_entry_point_under_graph_capture(oracle, n_tables):
     """The callers the entry point is for: recorded into a HIP graph (no allocation may happen
     there) and replayed with new ids in the same buffers, with eager calls of the same entry point
     between the replays (they share the built-in descriptor buffer, in stream order)."""
     rng = np.random.Generator(np.random.PCG64(31))
-    rows, dim, n_bags, n_ids = [700, 12000, 33], 64, 500, 6000
+    rows, dim, n_bags, n_ids = ([700, 12000, 33] + [211 + 37 * t for t in range(n_tables)])[:n_tables], 64, 500, 6000
     tables = [(rng.standard_normal((r, dim)) * 0.3).astype(np.float16) for r in rows]
     d_tab = [dev(t) for t in tables]
 
@@ -144,17 +196,17 @@ def test_no_alloc_entry_point_under_graph_capture(oracle):
     ids0, offs0 = batch(0)
     d_ids, d_off = [dev(i) for i in ids0], [dev(o) for o in offs0]
     desc = descriptors(d_tab, d_ids, d_off, dim)
-    out = torch.zeros((n_bags, 3 * dim), dtype=torch.float16, device="cuda")
-    x = ops._ext(d_tab[0], d_ids[0], torch.float16, out_row_stride=3 * dim)
+    out = torch.zeros((n_bags, n_tables * dim), dtype=torch.float16, device="cuda")
+    x = ops._ext(d_tab[0], d_ids[0], torch.float16, out_row_stride=n_tables * dim)
 
     def launch(dst):
         s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-        lib.check(lib.dll.fwdmi_embedding_bag_multi_noalloc(C.c_void_p(desc.ctypes.data), 3, n_bags,
+        lib.check(lib.dll.fwdmi_embedding_bag_multi_noalloc(C.c_void_p(desc.ctypes.data), n_tables, n_bags,
                                                             C.c_void_p(dst.data_ptr()), dim, 0, n_ids / float(n_bags),
                                                             C.byref(x), s))
 
     def want(ids, offs):
-        return np.concatenate([oracle.embedding_bag(tables[t], ids[t], offs[t], 0)[0] for t in range(3)], axis=1)
+        return np.concatenate([oracle.embedding_bag(tables[t], ids[t], offs[t], 0)[0] for t in range(n_tables)], axis=1)
 
     launch(out)                                     # eager first: the buffer's address is looked up here
     torch.cuda.synchronize()
@@ -166,7 +218,7 @@ def test_no_alloc_entry_point_under_graph_capture(oracle):
     other = torch.zeros_like(out)
     for seed in (1, 2, 3):
         ids, offs = batch(seed)
-        for t in range(3):
+        for t in range(n_tables):
             d_ids[t].copy_(dev(ids[t]))
             d_off[t].copy_(dev(offs[t]))
         out.fill_(-1.0)

@@ -137,6 +137,20 @@ SIGNATURES = {
     "fwdmi_plan_take_plugin": (_vp, [_vp, C.c_int]),
     "fwdmi_plan_meta": (_cp, [_vp]),
     "fwdmi_plan_close": (None, [_vp]),
+    "fwdmi_meta_new": (_vp, []),
+    "fwdmi_meta_load": (_vp, [_cp]),
+    "fwdmi_meta_parse": (_vp, [_cp]),
+    "fwdmi_plan_meta_data": (_vp, [_vp]),
+    "fwdmi_meta_save": (C.c_int, [_vp, _cp]),
+    "fwdmi_meta_json": (_cp, [_vp]),
+    "fwdmi_meta_infer_mode": (_i32, [_vp]),
+    "fwdmi_meta_opt_batch_size": (_i32, [_vp]),
+    "fwdmi_meta_max_batch_size": (_i32, [_vp]),
+    "fwdmi_meta_torch_module_path": (_cp, [_vp]),
+    "fwdmi_meta_unused_input_indices": (_i32, [_vp, C.POINTER(C.POINTER(_i32))]),
+    "fwdmi_meta_output_indices": (_i32, [_vp, C.POINTER(C.POINTER(_i32))]),
+    "fwdmi_meta_set": (C.c_int, [_vp, _i32, _i32, _i32, C.POINTER(_i32), _i32, C.POINTER(_i32), _i32, _cp]),
+    "fwdmi_meta_free": (None, [_vp]),
 }
 
 

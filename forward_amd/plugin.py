@@ -223,25 +223,109 @@ def getPluginRegistry():
     return PluginRegistry()
 
 
-# Keys of the reference's engine sidecar (source/trt_engine/trt_common/trt_meta_data.cpp:42-97).
-META_KEYS = ("infer_mode", "max_batch_size", "opt_batch_size", "output_indices", "unused_input_indices",
-             "torch_module_path")
+# InferMode of the reference (source/common/fwd_common.h:40-60): the sidecar stores the number.
+INFER_MODES = {"float": 0, "float32": 0, "half": 1, "float16": 1, "int8": 2, "int8_calib": 3}
+
+
+class EngineMetaData:
+    """The engine sidecar ``<engine file>.meta``, typed: mirror of the reference's ``EngineMetaData``
+    (source/trt_engine/trt_common/trt_meta_data.h:37-90, .cpp:42-97) over the library's reader and
+    writer.  ``infer_mode`` is an int (0 float, 1 half, 2 int8, 3 int8_calib), ``opt_batch_size`` /
+    ``max_batch_size`` ints, ``unused_input_indices`` a sorted list without repeats (a set in the
+    reference), ``output_indices`` a list, ``torch_module_path`` a string."""
+
+    KEYS = ("infer_mode", "max_batch_size", "opt_batch_size", "output_indices", "torch_module_path",
+            "unused_input_indices")
+
+    def __init__(self, infer_mode=0, opt_batch_size=-1, max_batch_size=-1, unused_input_indices=(),
+                 output_indices=(), torch_module_path=""):
+        if isinstance(infer_mode, str):
+            infer_mode = INFER_MODES[infer_mode]
+        self.infer_mode, self.opt_batch_size, self.max_batch_size = int(infer_mode), int(opt_batch_size), int(max_batch_size)
+        self.unused_input_indices = sorted(set(int(v) for v in unused_input_indices))
+        self.output_indices = [int(v) for v in output_indices]
+        self.torch_module_path = str(torch_module_path)
+
+    def __eq__(self, other):
+        return isinstance(other, EngineMetaData) and self.to_dict() == other.to_dict()
+
+    def __repr__(self):
+        return "EngineMetaData(%r)" % (self.to_dict(),)
+
+    def to_dict(self):
+        return {k: getattr(self, k) for k in self.KEYS}
+
+    @classmethod
+    def from_dict(cls, d):
+        """From a dict with the sidecar's keys, through the library's own reader: a missing key or
+        a value of the wrong type raises FwdmiError, as ``LoadMetaData`` returns false."""
+        import json
+        return cls._take(lib.dll.fwdmi_meta_parse(json.dumps(d).encode()))
+
+    @classmethod
+    def _take(cls, h):
+        if not h:
+            raise lib.FwdmiError(lib.ERR_BAD_ARG, lib.last_error())
+        h = C.c_void_p(h)
+        try:
+            def ints(fn):
+                p = C.POINTER(C.c_int32)()
+                n = fn(h, C.byref(p))
+                return [int(p[i]) for i in range(n)]
+            return cls(lib.dll.fwdmi_meta_infer_mode(h), lib.dll.fwdmi_meta_opt_batch_size(h),
+                       lib.dll.fwdmi_meta_max_batch_size(h), ints(lib.dll.fwdmi_meta_unused_input_indices),
+                       ints(lib.dll.fwdmi_meta_output_indices), lib.dll.fwdmi_meta_torch_module_path(h).decode())
+        finally:
+            lib.dll.fwdmi_meta_free(h)
+
+    def _handle(self):
+        h = C.c_void_p(lib.dll.fwdmi_meta_new())
+        u = (C.c_int32 * max(1, len(self.unused_input_indices)))(*self.unused_input_indices)
+        o = (C.c_int32 * max(1, len(self.output_indices)))(*self.output_indices)
+        lib.check(lib.dll.fwdmi_meta_set(h, self.infer_mode, self.opt_batch_size, self.max_batch_size, u,
+                                         len(self.unused_input_indices), o, len(self.output_indices),
+                                         self.torch_module_path.encode()))
+        return h
+
+    def to_json(self):
+        """The text ``SaveMetaData`` writes (keys in alphabetical order, four-space indentation)."""
+        h = self._handle()
+        try:
+            return lib.dll.fwdmi_meta_json(h).decode()
+        finally:
+            lib.dll.fwdmi_meta_free(h)
+
+    def SaveMetaData(self, meta_file):
+        h = self._handle()
+        try:
+            lib.check(lib.dll.fwdmi_meta_save(h, meta_file.encode()))
+        finally:
+            lib.dll.fwdmi_meta_free(h)
+        return True
+
+    @classmethod
+    def LoadMetaData(cls, meta_file):
+        return cls._take(lib.dll.fwdmi_meta_load(meta_file.encode()))
 
 
 def save_plan(path, layers, meta=None):
-    """Writes ``layers`` = [(layer_name, Plugin), ...] to ``path`` and ``meta`` (a dict with the
-    reference's sidecar keys) to ``path + ".meta"``: the plugin part of ``TrtForwardEngine::Save``."""
+    """Writes ``layers`` = [(layer_name, Plugin), ...] to ``path`` and ``meta`` (an EngineMetaData, or
+    a dict with the sidecar's keys and types) to ``path + ".meta"``: the plugin part of
+    ``TrtForwardEngine::Save``.  A ``meta`` the reference's reader would reject raises FwdmiError
+    and nothing is written."""
     import json
     n = len(layers)
     handles = (C.c_void_p * max(1, n))(*[p._h for _, p in layers])
     names = (C.c_char_p * max(1, n))(*[name.encode() for name, _ in layers])
+    if isinstance(meta, EngineMetaData):
+        meta = meta.to_dict()
     text = None if meta is None else json.dumps(meta).encode()
     lib.check(lib.dll.fwdmi_plan_save(path.encode(), handles, names, n, text))
 
 
 def load_plan(path):
-    """Returns ``([(layer_name, Plugin), ...], meta_dict)``: the plugin part of ``TrtForwardEngine::Load``."""
-    import json
+    """Returns ``([(layer_name, Plugin), ...], EngineMetaData or None)``: the plugin part of
+    ``TrtForwardEngine::Load``.  A sidecar that is present but malformed fails the load."""
     h = lib.dll.fwdmi_plan_load(path.encode())
     if not h:
         raise lib.FwdmiError(lib.ERR_TRUNCATED, lib.last_error())
@@ -249,7 +333,8 @@ def load_plan(path):
     try:
         layers = [(lib.dll.fwdmi_plan_layer_name(h, i).decode(), Plugin(lib.dll.fwdmi_plan_take_plugin(h, i)))
                   for i in range(lib.dll.fwdmi_plan_size(h))]
-        text = lib.dll.fwdmi_plan_meta(h).decode()
+        m = lib.dll.fwdmi_plan_meta_data(h)
+        meta = EngineMetaData._take(m) if m else None
     finally:
         lib.dll.fwdmi_plan_close(h)
-    return layers, (json.loads(text) if text else {})
+    return layers, meta

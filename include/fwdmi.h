@@ -382,26 +382,60 @@ int fwdmi_plugin_take_oob_flag(fwdmi_plugin* p, void* stream);
  *  3. Plan files: the plugins of an engine in one file + the "<file>.meta" JSON sidecar
  *     replaces the plugin part of TrtForwardEngine::Save / Load
  *     (source/trt_engine/trt_engine/trt_fwd_engine.cpp:156-209) and the sidecar of
- *     source/trt_engine/trt_common/trt_meta_data.cpp:42-97 (keys infer_mode, max_batch_size,
- *     opt_batch_size, output_indices, unused_input_indices, torch_module_path; the text is
- *     stored as given).
+ *     source/trt_engine/trt_common/trt_meta_data.cpp:42-97: keys infer_mode (int, the InferMode of
+ *     source/common/fwd_common.h:40-46: 0 float, 1 half, 2 int8, 3 int8_calib), opt_batch_size,
+ *     max_batch_size (ints), unused_input_indices, output_indices (int arrays), torch_module_path
+ *     (string), written in the reference's text form so that either side loads the other's file.
  * ========================================================================================= */
 typedef struct fwdmi_plan fwdmi_plan;
 
 /* Serializes n plugins (with the layer names they were created under) into `path`;
- * meta_json (may be NULL) goes to "<path>.meta". */
+ * meta_json (may be NULL) is checked as a sidecar (every key above present with its type, else
+ * FWDMI_ERR_BAD_ARG and nothing is written) and goes to "<path>.meta" in the reference's form. */
 int fwdmi_plan_save(const char* path, fwdmi_plugin* const* plugins, const char* const* layer_names, int n,
                     const char* meta_json);
 /* Reads a plan back: every entry is re-created through its registered creator's
- * deserializePlugin.  NULL on a missing / truncated file or an unknown (type, version). */
+ * deserializePlugin.  NULL on a missing / truncated file, an unknown (type, version) or a sidecar
+ * that is present but malformed (a plan without a sidecar loads, with no settings). */
 fwdmi_plan* fwdmi_plan_load(const char* path);
 int fwdmi_plan_size(fwdmi_plan* plan);
 const char* fwdmi_plan_layer_name(fwdmi_plan* plan, int i);
 /* Hands entry i to the caller (who destroys it); a second call for the same i returns NULL. */
 fwdmi_plugin* fwdmi_plan_take_plugin(fwdmi_plan* plan, int i);
-/* Text of "<path>.meta" ("" if the sidecar is absent). */
+/* The sidecar as JSON text in the reference's form ("" if the sidecar is absent). */
 const char* fwdmi_plan_meta(fwdmi_plan* plan);
 void fwdmi_plan_close(fwdmi_plan* plan);
+
+/* The sidecar by itself, typed: EngineMetaData of source/trt_engine/trt_common/trt_meta_data.h:37-90.
+ * A new object holds the reference's defaults (infer_mode 0, batch sizes -1, empty arrays and path). */
+typedef struct fwdmi_meta fwdmi_meta;
+fwdmi_meta* fwdmi_meta_new(void);
+/* EngineMetaData::LoadMetaData, trt_meta_data.cpp:49-79.  NULL when the file cannot be opened, is
+ * not JSON, lacks infer_mode / opt_batch_size / max_batch_size / torch_module_path or holds a
+ * value of the wrong type (fwdmi_last_error says which); absent index arrays read as empty. */
+fwdmi_meta* fwdmi_meta_load(const char* meta_file);
+/* The same from JSON text. */
+fwdmi_meta* fwdmi_meta_parse(const char* json_text);
+/* A copy of a loaded plan's sidecar; NULL if the plan has none.  Freed with fwdmi_meta_free. */
+fwdmi_meta* fwdmi_plan_meta_data(fwdmi_plan* plan);
+/* EngineMetaData::SaveMetaData, trt_meta_data.cpp:81-97: keys in alphabetical order, four-space
+ * indentation, one array element per line, trailing newline. */
+int fwdmi_meta_save(fwdmi_meta* m, const char* meta_file);
+/* The text fwdmi_meta_save writes (valid until the next call on `m`). */
+const char* fwdmi_meta_json(fwdmi_meta* m);
+int32_t fwdmi_meta_infer_mode(fwdmi_meta* m);
+int32_t fwdmi_meta_opt_batch_size(fwdmi_meta* m);
+int32_t fwdmi_meta_max_batch_size(fwdmi_meta* m);
+const char* fwdmi_meta_torch_module_path(fwdmi_meta* m);
+/* Element count; *data (may be NULL) points at the elements, ascending for the unused inputs
+ * (a set in the reference), valid until the next call of the same getter on `m`. */
+int32_t fwdmi_meta_unused_input_indices(fwdmi_meta* m, const int32_t** data);
+int32_t fwdmi_meta_output_indices(fwdmi_meta* m, const int32_t** data);
+/* Sets every member at once (arrays are copied; torch_module_path NULL = ""). */
+int fwdmi_meta_set(fwdmi_meta* m, int32_t infer_mode, int32_t opt_batch_size, int32_t max_batch_size,
+                   const int32_t* unused_input_indices, int32_t n_unused, const int32_t* output_indices,
+                   int32_t n_outputs, const char* torch_module_path);
+void fwdmi_meta_free(fwdmi_meta* m);
 
 #ifdef __cplusplus
 }

@@ -11,7 +11,8 @@ from forward_amd import lib, plugin
 from forward_amd.plugin import PluginFieldData as F
 
 REG = plugin.getPluginRegistry()
-META = {"infer_mode": "float16", "max_batch_size": 65536, "opt_batch_size": 65536, "output_indices": [0],
+# infer_mode is the number of the reference's InferMode (1 = half), as trt_meta_data.cpp:60,83 reads and writes it
+META = {"infer_mode": 1, "max_batch_size": 65536, "opt_batch_size": 65536, "output_indices": [0],
         "unused_input_indices": [], "torch_module_path": "dlrm.pth"}
 
 
@@ -40,8 +41,22 @@ def test_plan_roundtrip_and_sidecar(tmp_path):
     raw = open(path, "rb").read()
     assert raw[:8] == b"FWDMIPL1" and struct.unpack("<I", raw[8:12]) == (3,)
     assert json.load(open(path + ".meta")) == META           # keys of trt_meta_data.cpp:42-97
+    # the very bytes the reference's JSON library writes for these members (tests/golden/meta/)
+    assert open(path + ".meta", "rb").read() == open(os.path.join(os.path.dirname(__file__), "golden", "meta",
+                                                                  "dlrm_half.meta"), "rb").read()
     loaded, meta = plugin.load_plan(path)
-    assert meta == META and [n for n, _ in loaded] == [n for n, _ in layers]
+    assert meta.to_dict() == META and [n for n, _ in loaded] == [n for n, _ in layers]
+    # a sidecar the reference's reader rejects is refused before anything is written, and fails a load
+    with pytest.raises(lib.FwdmiError, match="infer_mode"):
+        plugin.save_plan(str(tmp_path / "bad.plan"), layers, dict(META, infer_mode="float16"))
+    assert not os.path.exists(str(tmp_path / "bad.plan"))
+    good_meta = open(path + ".meta").read()
+    open(path + ".meta", "w").write(good_meta.replace('"max_batch_size": 65536', '"max_batch_size": "many"'))
+    with pytest.raises(lib.FwdmiError, match="max_batch_size"):
+        plugin.load_plan(path)
+    os.remove(path + ".meta")
+    assert plugin.load_plan(path)[1] is None                 # no sidecar: a plan without engine settings
+    open(path + ".meta", "w").write(good_meta)
     for (_, a), (_, b) in zip(layers, loaded):
         assert (a.getPluginType(), a.getPluginVersion(), a.getPluginNamespace()) == \
                (b.getPluginType(), b.getPluginVersion(), b.getPluginNamespace())

@@ -2,8 +2,11 @@
 
 Counterpart of the reference's torch-side glue (``TorchEngine::ParseInput`` / ``CopyFromBuffers``,
 source/fwd_torch/torch_engine/torch_engine.cpp:134-174): there, int64 ids are copied to int32 and
-outputs are copied out of engine buffers; here the ops consume int32 or int64 ids as they are and
-write straight into the tensors they return.  ``nn.EmbeddingBag`` / ``nn.Embedding`` modules of an
+outputs are copied out of engine buffers; here the bag ops consume int32 or int64 ids as they are and
+write straight into the tensors they return, or, in their ``*_out`` forms, into tensors the caller
+supplies (declared to PyTorch as mutated arguments), so that a serving loop reuses its buffers.
+The BERT ops (``emb_layer_norm``, ``emb_skip_layer_norm``) take the ``[B, S]`` tensors a PyTorch model
+holds (``batch_major``) or the plugin's ``[S, B]``.  ``nn.EmbeddingBag`` / ``nn.Embedding`` modules of an
 inference model can be swapped for the HIP path with ``replace_embedding_modules``.
 """
 from typing import List, Optional
@@ -82,6 +85,122 @@ def skip_layer_norm(x: torch.Tensor, skip: Optional[torch.Tensor], gamma: torch.
 @skip_layer_norm.register_fake
 def _(x, skip, gamma, beta, bias, eps):
     return torch.empty_like(x)
+
+
+def _i32(t):
+    """ids of the BERT ops: the launchers read int32 (int64 ids are narrowed, as the reference's
+    ParseInput does for every integer input, torch_engine.cpp:134-140)."""
+    return None if t is None else t.to(torch.int32).contiguous()
+
+
+def _f32(t):
+    return None if t is None else t.float().contiguous()
+
+
+@torch.library.custom_op("fwdmi::emb_layer_norm", mutates_args=())
+def emb_layer_norm(input_ids: torch.Tensor, segment_ids: torch.Tensor, input_mask: Optional[torch.Tensor],
+                   word: torch.Tensor, pos: torch.Tensor, tok: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor,
+                   eps: float, batch_major: bool) -> List[torch.Tensor]:
+    """BERT embedding + LayerNorm: ``[out, mask_idx]``.  ids / mask are ``[B, S]`` with ``batch_major``
+    (out ``[B, S, H]``), else the plugin's ``[S, B]`` (out ``[S, B, H]``); ``mask_idx`` is int32 ``[B]``
+    (empty without a mask)."""
+    out, midx = ops.emb_layer_norm(_i32(input_ids), _i32(segment_ids), _i32(input_mask), word, pos, tok, _f32(gamma),
+                                   _f32(beta), eps=eps, batch_major=batch_major)
+    return [out, midx if midx is not None else torch.empty((0,), dtype=torch.int32, device=out.device)]
+
+
+@emb_layer_norm.register_fake
+def _(input_ids, segment_ids, input_mask, word, pos, tok, gamma, beta, eps, batch_major):
+    b = input_ids.shape[0] if batch_major else input_ids.shape[1]
+    return [word.new_empty(tuple(input_ids.shape) + (word.shape[1],)),
+            input_ids.new_empty((b if input_mask is not None else 0,), dtype=torch.int32)]
+
+
+@torch.library.custom_op("fwdmi::emb_skip_layer_norm", mutates_args=())
+def emb_skip_layer_norm(input_ids: torch.Tensor, segment_ids: torch.Tensor, input_mask: Optional[torch.Tensor],
+                        word: torch.Tensor, pos: torch.Tensor, tok: torch.Tensor, gamma: torch.Tensor,
+                        beta: torch.Tensor, eps: float, skip: torch.Tensor, gamma2: torch.Tensor, beta2: torch.Tensor,
+                        bias2: Optional[torch.Tensor], eps2: float, batch_major: bool) -> List[torch.Tensor]:
+    """The embedding stage and the SkipLayerNorm that consumes it in one launch:
+    ``out = LN2(LN(word + pos + tok) + skip (+ bias2))``, equal bit for bit to the two ops in a row."""
+    out, midx = ops.emb_layer_norm(_i32(input_ids), _i32(segment_ids), _i32(input_mask), word, pos, tok, _f32(gamma),
+                                   _f32(beta), eps=eps, batch_major=batch_major, skip=skip.contiguous(),
+                                   gamma2=_f32(gamma2), beta2=_f32(beta2), bias2=_f32(bias2), eps2=eps2)
+    return [out, midx if midx is not None else torch.empty((0,), dtype=torch.int32, device=out.device)]
+
+
+@emb_skip_layer_norm.register_fake
+def _(input_ids, segment_ids, input_mask, word, pos, tok, gamma, beta, eps, skip, gamma2, beta2, bias2, eps2, batch_major):
+    b = input_ids.shape[0] if batch_major else input_ids.shape[1]
+    return [word.new_empty(tuple(input_ids.shape) + (word.shape[1],)),
+            input_ids.new_empty((b if input_mask is not None else 0,), dtype=torch.int32)]
+
+
+# ---- forms that write into the caller's tensors ------------------------------------------------
+# Where the reference copies every output out of an engine buffer into a fresh tensor
+# (TorchEngine::CopyFromBuffers, torch_engine.cpp:150-174), these write the result where the caller
+# wants it; PyTorch is told which argument is written (mutates_args), nothing is returned.
+
+@torch.library.custom_op("fwdmi::embedding_bag_out", mutates_args=("out",))
+def embedding_bag_out(out: torch.Tensor, weight: torch.Tensor, indices: torch.Tensor, offsets: torch.Tensor, mode: int,
+                      per_sample_weights: Optional[torch.Tensor], include_last_offset: bool, out_col: int) -> None:
+    """``out[:, out_col : out_col + dim]`` = the bags; ``out`` is ``[n_bags, W]`` of the table's dtype."""
+    ops.embedding_bag(weight, indices.contiguous(), offsets.contiguous().to(indices.dtype), mode,
+                      per_sample_weights=per_sample_weights, include_last_offset=include_last_offset, out=out,
+                      out_col=out_col, out_dtype=out.dtype)
+
+
+@torch.library.custom_op("fwdmi::embedding_bag_group_out", mutates_args=("out",))
+def embedding_bag_group_out(out: torch.Tensor, weights: List[torch.Tensor], indices: List[torch.Tensor],
+                            offsets: List[torch.Tensor], mode: int, include_last_offset: bool,
+                            per_sample_weights: List[Optional[torch.Tensor]]) -> None:
+    idt = indices[0].dtype
+    psw = [None if w is None else w.to(weights[0].dtype).contiguous() for w in per_sample_weights]
+    if all(w is None for w in psw):
+        psw = None
+    ops.embedding_bag_group(weights, [i.contiguous() for i in indices], [o.contiguous().to(idt) for o in offsets], mode,
+                            include_last_offset=include_last_offset, per_sample_weights=psw, out=out, out_dtype=out.dtype)
+
+
+@torch.library.custom_op("fwdmi::skip_layer_norm_out", mutates_args=("out",))
+def skip_layer_norm_out(out: torch.Tensor, x: torch.Tensor, skip: Optional[torch.Tensor], gamma: torch.Tensor,
+                        beta: torch.Tensor, bias: Optional[torch.Tensor], eps: float) -> None:
+    """``out``: a tensor of ``x``'s shape and dtype (not ``x`` or ``skip`` themselves)."""
+    ops.skip_layer_norm(x.contiguous(), _f32(gamma), _f32(beta), skip=None if skip is None else skip.contiguous(),
+                        bias=_f32(bias), eps=eps, out=out)
+
+
+@torch.library.custom_op("fwdmi::emb_layer_norm_out", mutates_args=("out", "mask_idx"))
+def emb_layer_norm_out(out: torch.Tensor, mask_idx: Optional[torch.Tensor], input_ids: torch.Tensor,
+                       segment_ids: torch.Tensor, input_mask: Optional[torch.Tensor], word: torch.Tensor,
+                       pos: torch.Tensor, tok: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, eps: float,
+                       skip: Optional[torch.Tensor], gamma2: Optional[torch.Tensor], beta2: Optional[torch.Tensor],
+                       bias2: Optional[torch.Tensor], eps2: float, batch_major: bool) -> None:
+    """Both BERT forms (``skip`` given: the fused embedding + SkipLayerNorm) into ``out`` / ``mask_idx``."""
+    ops.emb_layer_norm(_i32(input_ids), _i32(segment_ids), _i32(input_mask), word, pos, tok, _f32(gamma), _f32(beta),
+                       eps=eps, batch_major=batch_major, out=out, mask_idx=mask_idx,
+                       skip=None if skip is None else skip.contiguous(), gamma2=_f32(gamma2), beta2=_f32(beta2),
+                       bias2=_f32(bias2), eps2=eps2)
+
+
+class BertEmbeddings(torch.nn.Module):
+    """Inference replacement of a BERT embedding block (word + position + token-type lookup, then
+    LayerNorm) on ``[B, S]`` tensors: ``forward(input_ids, token_type_ids, attention_mask)`` returns
+    ``(embeddings [B, S, H], valid_length int32 [B])``, the two outputs of the embedding plugin the
+    reference wires in (trt_bert_creator.h:113-155), without its transposes to and from ``[S, B]``."""
+
+    def __init__(self, word, pos, tok, gamma, beta, eps=1e-12):
+        super().__init__()
+        p = lambda t: torch.nn.Parameter(t.detach().contiguous(), requires_grad=False)
+        self.word, self.pos, self.tok = p(word), p(pos), p(tok)
+        self.gamma, self.beta, self.eps = p(gamma.float()), p(beta.float()), float(eps)
+
+    def forward(self, input_ids, token_type_ids=None, attention_mask=None):
+        if token_type_ids is None:
+            token_type_ids = torch.zeros_like(input_ids)
+        out, midx = torch.ops.fwdmi.emb_layer_norm(input_ids, token_type_ids, attention_mask, self.word, self.pos,
+                                                   self.tok, self.gamma, self.beta, self.eps, True)
+        return out, midx
 
 
 class EmbeddingBag(torch.nn.Module):

@@ -100,3 +100,102 @@ def test_collection_is_the_concatenation_of_its_bags(kats):
     mixed = [torch.nn.EmbeddingBag(5, 4, mode="sum"), torch.nn.EmbeddingBag(5, 4, mode="mean")]
     with pytest.raises(ValueError):
         torch_ops.EmbeddingBagCollection.from_torch(mixed)
+
+
+def _bert_inputs(wl):
+    """[B, S] tensors as a PyTorch model holds them (int64 ids), plus the plugin-layout originals."""
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    bs = lambda a: dev(a.T).long()
+    return (bs(wl.input_ids), bs(wl.segment_ids), bs(wl.input_mask), dev(wl.word), dev(wl.pos), dev(wl.tok),
+            dev(wl.gamma.astype(np.float32)), dev(wl.beta.astype(np.float32)))
+
+
+@pytest.mark.parametrize("cfg", ["config3", "config5"])
+def test_bert_ops_against_the_oracle(oracle, cfg):
+    """torch.ops.fwdmi.emb_layer_norm / emb_skip_layer_norm on [B, S] int64 tensors (scaled configs 3 and 5)
+    against the oracle: fp16 abs 1e-2 / rel 5e-3, mask index exact; the fused op equal to the two ops in a row."""
+    wl = workloads.config3(variant=4, batch=5, seq=48) if cfg == "config3" else workloads.config5(variant=4, batch=3, seq=96)
+    ids, seg, msk, word, pos, tok, g, b = _bert_inputs(wl)
+    out, midx = torch.ops.fwdmi.emb_layer_norm(ids, seg, msk, word, pos, tok, g, b, wl.eps, True)
+    want, want_midx, _ = oracle.emb_layer_norm(wl.input_ids, wl.segment_ids, wl.input_mask, wl.word, wl.pos, wl.tok,
+                                               wl.gamma, wl.beta, eps=wl.eps)
+    assert out.shape == (ids.shape[0], ids.shape[1], wl.word.shape[1]) and out.dtype == torch.float16
+    np.testing.assert_allclose(out.float().cpu().numpy().transpose(1, 0, 2), want.astype(np.float32), atol=1e-2, rtol=5e-3)
+    assert np.array_equal(midx.cpu().numpy(), want_midx) and np.array_equal(want_midx, wl.valid_len)
+    # the plugin's own [S, B] layout through the same op
+    out_sb, midx_sb = torch.ops.fwdmi.emb_layer_norm(ids.T.contiguous(), seg.T.contiguous(), msk.T.contiguous(), word, pos,
+                                                     tok, g, b, wl.eps, False)
+    assert torch.equal(out_sb.transpose(0, 1), out) and torch.equal(midx_sb, midx)
+    # without a mask: no mask index
+    _, none = torch.ops.fwdmi.emb_layer_norm(ids, seg, None, word, pos, tok, g, b, wl.eps, True)
+    assert none.numel() == 0
+    # into the caller's tensors
+    out2, midx2 = torch.full_like(out, 7.0), torch.full_like(midx, -1)
+    torch.ops.fwdmi.emb_layer_norm_out(out2, midx2, ids, seg, msk, word, pos, tok, g, b, wl.eps, None, None, None, None,
+                                       0.0, True)
+    assert torch.equal(out2, out) and torch.equal(midx2, midx)
+    mod = torch_ops.BertEmbeddings(word, pos, tok, g, b, wl.eps)
+    m_out, m_len = mod(ids, seg, msk)
+    assert torch.equal(m_out, out) and torch.equal(m_len, midx)
+    if wl.skip is None:
+        return
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    skip = dev(wl.skip.transpose(1, 0, 2))
+    g2, b2, bi2 = (dev(a.astype(np.float32)) for a in (wl.skip_gamma, wl.skip_beta, wl.skip_bias))
+    fused, fmidx = torch.ops.fwdmi.emb_skip_layer_norm(ids, seg, msk, word, pos, tok, g, b, wl.eps, skip, g2, b2, bi2,
+                                                       wl.eps, True)
+    chained = torch.ops.fwdmi.skip_layer_norm(out, skip, g2, b2, bi2, wl.eps)
+    assert torch.equal(fused, chained) and torch.equal(fmidx, midx)
+    want2 = oracle.skip_layer_norm(want, wl.skip_gamma, wl.skip_beta, skip=wl.skip, bias=wl.skip_bias, eps=wl.eps)
+    np.testing.assert_allclose(fused.float().cpu().numpy().transpose(1, 0, 2), want2.astype(np.float32), atol=1e-2, rtol=5e-3)
+    buf = torch.zeros_like(fused)
+    torch.ops.fwdmi.emb_layer_norm_out(buf, None, ids, seg, msk, word, pos, tok, g, b, wl.eps, skip, g2, b2, bi2, wl.eps, True)
+    assert torch.equal(buf, fused)
+    buf.zero_()
+    torch.ops.fwdmi.skip_layer_norm_out(buf, out, skip, g2, b2, bi2, wl.eps)
+    assert torch.equal(buf, chained)
+
+
+def test_out_forms_write_into_the_callers_tensors(kats, oracle):
+    """*_out ops: declared to PyTorch as mutating `out`, results equal to the returning forms; on the reference's
+    DLRM case (test_torch_dlrm.h:34-57) and on a larger stage, against the oracle."""
+    d = kats["dlrm"]
+    ws = [torch.tensor(np.array(t, np.float32), device="cuda") for t in d["tables"]]
+    idx = [torch.tensor(i, device="cuda") for i in d["indices"]]
+    off = [torch.tensor(o, device="cuda") for o in d["offsets"]]
+    out = torch.full((2, 6), 9.0, device="cuda")
+    for t in range(3):
+        torch.ops.fwdmi.embedding_bag_out(out, ws[t], idx[t], off[t], 0, None, False, 2 * t)
+    expect = np.concatenate([[[0.48071694, 0.18480009], [0.41585842, -0.29087239]],
+                             [[-0.18103497, 0.26449448], [-0.25194445, -0.24395032]],
+                             [[-0.44896644, -0.45899662], [-0.44896644, -0.45899662]]], axis=1)
+    np.testing.assert_allclose(out.cpu().numpy(), expect, atol=1e-6)           # test_torch_dlrm.h:56
+    out2 = torch.full((2, 6), 9.0, device="cuda")
+    torch.ops.fwdmi.embedding_bag_group_out(out2, ws, idx, off, 0, False, [None] * 3)
+    assert torch.equal(out2, out)
+    assert "Tensor(a0!) out" in str(torch.ops.fwdmi.embedding_bag_out.default._schema)
+    assert "Tensor(a0!) out" in str(torch.ops.fwdmi.embedding_bag_group_out.default._schema)
+
+    wl = workloads.config4(variant=3, n_tables=5, n_bags=2000, max_rows=30000)
+    tabs = [wl.host_table(t) for t in range(5)]
+    ws = [torch.from_numpy(t).cuda() for t in tabs]
+    ids = [torch.from_numpy(i.astype(np.int64)).cuda() for i in wl.indices]
+    offs = [torch.from_numpy(o.astype(np.int64)).cuda() for o in wl.offsets]
+    want = np.zeros((2000, 5 * 128), np.float16)
+    for t in range(5):
+        oracle.embedding_bag(tabs[t], wl.indices[t], wl.offsets[t], oracle.OP_SUM, out=want, out_col=128 * t)
+    buf = torch.zeros((2000, 5 * 128), dtype=torch.float16, device="cuda")
+    torch.ops.fwdmi.embedding_bag_group_out(buf, ws, ids, offs, 0, False, [None] * 5)
+    assert np.array_equal(buf.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    buf.zero_()
+    for t in range(5):
+        torch.ops.fwdmi.embedding_bag_out(buf, ws[t], ids[t], offs[t], 0, None, False, 128 * t)
+    assert np.array_equal(buf.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # PyTorch's own checks of a custom op: schema (which arguments are written) and shape inference
+    torch.library.opcheck(torch.ops.fwdmi.embedding_bag_out.default, (buf, ws[0], ids[0], offs[0], 0, None, False, 0),
+                          test_utils=("test_schema",))
+    ids3, seg3 = torch.zeros((2, 4), dtype=torch.int64, device="cuda"), torch.zeros((2, 4), dtype=torch.int64, device="cuda")
+    word = torch.randn(10, 64, device="cuda", dtype=torch.float16)
+    args = (ids3, seg3, torch.ones_like(ids3), word, word[:4].clone(), word[:2].clone(), torch.ones(64, device="cuda"),
+            torch.zeros(64, device="cuda"), 1e-12, True)
+    torch.library.opcheck(torch.ops.fwdmi.emb_layer_norm.default, args, test_utils=("test_schema", "test_faketensor"))

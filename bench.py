@@ -75,6 +75,12 @@ def parse():
     ap.add_argument("--ids", default="zipf", choices=["zipf", "equal", "uniform"],
                     help="--replay only: keep the workload's ids, or replace them (lengths kept) by one row per "
                          "table / by uniform random rows")
+    ap.add_argument("--order", default="stream", choices=["stream", "phased", "phased_unsorted", "bursts", "grouped"],
+                    help="--replay only: the order of the ids inside every workgroup's chunk: as they come; the ids "
+                         "that occur once in the chunk first and the repeated ones after them, all slots in the same "
+                         "phase at the same time (likely misses apart from likely hits; phased_unsorted: the repeated "
+                         "ones in their original order, phased: sorted by row); bursts: no phases, but the repeated "
+                         "ids sorted among themselves, so that equal rows are fetched together; or all sorted by row")
     ap.add_argument("--lru-sim", action="store_true",
                     help="no GPU: rows fetched by an LRU cache of one XCD's L2 size over each table's id stream "
                          "(the floor of the re-fetch ratio for table-at-a-time processing)")
@@ -470,6 +476,21 @@ def hbm_gather(torch, ops, copy_gbs=None, rows=1 << 24, dim=128, n_bags=262144, 
         n[0] += 1
     _, per = time_events(torch, fn, steps, 5)
     ms = float(np.mean(per))
+    # the same table read front to back by a kernel that does nothing else: what contiguous reads get from HBM here
+    read_gbs = None
+    dll = microbench_dll()
+    if dll is not None:
+        import ctypes as C
+        dll.fwdmi_mb_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+        nbytes_tab = table.numel() * 2
+        grid = torch.cuda.get_device_properties(0).multi_processor_count * 8
+
+        def rd():
+            rc = dll.fwdmi_mb_stream_read(table.data_ptr(), nbytes_tab, grid, torch.cuda.current_stream().cuda_stream)
+            if rc:
+                raise RuntimeError("stream read failed: hipError %d" % rc)
+        _, per_r = time_events(torch, rd, 10, 3)
+        read_gbs = nbytes_tab / (float(np.mean(per_r)) * 1e-3) / 1e9
     nbytes = n_bags * bag_len * (dim * 2 + 4) + n_bags * 4 + n_bags * dim * 2
     res = {"what": "uniform random ids over a 4 GiB fp16 table (2^24 rows x 128): %d bags x %d ids per launch, sum"
                    % (n_bags, bag_len),
@@ -479,6 +500,10 @@ def hbm_gather(torch, ops, copy_gbs=None, rows=1 << 24, dim=128, n_bags=262144, 
     if copy_gbs:
         res["device_copy_GBs"] = copy_gbs
         res["over_device_copy_rate"] = res["algorithmic_GBs"] / copy_gbs
+    if read_gbs:
+        res["contiguous_read_GBs"] = read_gbs
+        res["contiguous_read_is"] = "the same 4 GiB table read front to back with 128-bit loads by a kernel that does nothing else"
+        res["over_contiguous_read_rate"] = res["algorithmic_GBs"] / read_gbs
     return res
 
 
@@ -653,6 +678,9 @@ def mixed_bag_lengths(torch, ops, workloads, wl, tabs):
     return res
 
 
+REPLAY_CHUNK = 1830                   # ids per replay workgroup, as the product's runs of 112 bags x 16.3 ids
+
+
 def replay_times(torch, ops, wl, tabs, idx, off, steps=60):
     """Times (ms, median of HIP-event durations) of bench_aux/replay_gather.hip on the
     workload's id stream: the rows alone, the rows plus as many stored bytes as the product writes
@@ -662,7 +690,7 @@ def replay_times(torch, ops, wl, tabs, idx, off, steps=60):
     dll = microbench_dll()
     if dll is None:
         return None
-    chunk = 2600                      # ids per workgroup, as the product's runs of 160 bags x 16.3 ids
+    chunk = REPLAY_CHUNK
     it_t, it_s, it_c = [], [], []
     for t in range(len(wl.rows)):
         n = wl.indices[t].size
@@ -703,7 +731,35 @@ def replay_times(torch, ops, wl, tabs, idx, off, steps=60):
     return res
 
 
-def replay(torch, ops, workloads, ids_mode):
+def reorder_chunks(ids, chunk, order):
+    """The id stream of one table with every `chunk` ids (what one replay workgroup fetches)
+    rearranged.  "phased": the ids that occur once in the chunk, then the repeated ones sorted by row,
+    dealt to the sixteen slots of the workgroup in turn so that all slots fetch once-only rows
+    (likely misses) at the same time and repeated rows (likely hits) at the same time;
+    "phased_unsorted": the same two phases with the repeated ids in their original order; "bursts":
+    every id stays where a once-only or a repeated id was, but the repeated ones are sorted among
+    themselves (equal rows are fetched together, misses and hits stay mixed); "grouped": sorted by row."""
+    out = np.empty_like(ids)
+    for s0 in range(0, ids.size, chunk):
+        c = ids[s0:s0 + chunk]
+        if order == "grouped":
+            o = np.sort(c)
+        else:
+            _, inv, cnt = np.unique(c, return_inverse=True, return_counts=True)
+            once = cnt[inv] == 1
+            if order == "phased":
+                o = np.concatenate([c[once], np.sort(c[~once])])
+            elif order == "phased_unsorted":
+                o = np.concatenate([c[once], c[~once]])
+            else:   # bursts
+                o = c.copy()
+                o[~once] = np.sort(c[~once])
+        # slot k of the workgroup sums a contiguous sixteenth of the chunk: give it elements k, k+16, ... of `o`
+        out[s0:s0 + c.size] = np.concatenate([o[k::16] for k in range(16)])
+    return out
+
+
+def replay(torch, ops, workloads, ids_mode, order="stream"):
     """`--replay`: the product launch beside the bag-free replay of the same id stream (a table on stdout)."""
     wl = workloads.config4()
     rng = np.random.Generator(np.random.PCG64(1))
@@ -725,10 +781,17 @@ def replay(torch, ops, workloads, ids_mode):
     print("%-72s %8.4f ms" % ("product launch (bags, ordered by length, %d result rows of 256 B)" %
                               (wl.n_bags * len(wl.rows)), float(np.median(per))), flush=True)
     del out, batch
+    if order != "stream":
+        # the replay knows no bags, so the order inside a workgroup's chunk is free: the product launch above
+        # ran on the ids as they come, the replay below runs on the rearranged stream (the same rows in all)
+        t0 = time.time()
+        idx = [torch.from_numpy(reorder_chunks(i, REPLAY_CHUNK, order)).cuda() for i in wl.indices]
+        print("ids inside every chunk of %d rearranged (%s) in %.1f s" % (REPLAY_CHUNK, order, time.time() - t0), flush=True)
     r = replay_times(torch, ops, wl, tabs, idx, off)
     if r is None:
         raise SystemExit("build the measurement aid first: make -C bench_aux")
     e = r["rows_per_result_row"]
+    print("replay, ids inside a chunk: %s" % order)
     for label, key in (("gather only (one result row per slot)", "gather_only_ms"),
                        ("gather + a 256 B result row every %d rows, plain stores" % e, "gather_plain_stores_ms"),
                        ("gather + a 256 B result row every %d rows, non-temporal stores" % e, "gather_streaming_stores_ms"),
@@ -788,7 +851,7 @@ def main():
         sweep_layer_norm(torch, ops)
         return
     if args.replay:
-        replay(torch, ops, workloads, args.ids)
+        replay(torch, ops, workloads, args.ids, args.order)
         return
 
     t0 = time.time()

@@ -81,6 +81,9 @@ def parse():
                          "phase at the same time (likely misses apart from likely hits; phased_unsorted: the repeated "
                          "ones in their original order, phased: sorted by row); bursts: no phases, but the repeated "
                          "ids sorted among themselves, so that equal rows are fetched together; or all sorted by row")
+    ap.add_argument("--hot", type=int, default=0, metavar="K",
+                    help="--replay only: also replay with the K (at most 64) most frequent rows of every table served "
+                         "from LDS instead of through the L1 (the split of every chunk done on the host: an upper bound)")
     ap.add_argument("--lru-sim", action="store_true",
                     help="no GPU: rows fetched by an LRU cache of one XCD's L2 size over each table's id stream "
                          "(the floor of the re-fetch ratio for table-at-a-time processing)")
@@ -759,7 +762,72 @@ def reorder_chunks(ids, chunk, order):
     return out
 
 
-def replay(torch, ops, workloads, ids_mode, order="stream"):
+def replay_hot_times(torch, ops, wl, tabs, k_hot, steps=60):
+    """bench_aux/replay_hot.hip on the workload's id stream: every chunk rearranged on the host into the
+    ids of rows that are not among the table's `k_hot` most frequent ones (counted on this batch) and,
+    behind them, one LDS slot number per fetch of a hot row.  Returns ms (median of HIP-event
+    durations) without and with result stores, and the share of the fetches that LDS serves."""
+    import ctypes as C
+    dll = microbench_dll()
+    if dll is None:
+        return None
+    chunk = REPLAY_CHUNK
+    it_t, it_s, it_c, it_h, streams, hots = [], [], [], [], [], []
+    n_hot_fetches = 0
+    for t in range(len(wl.rows)):
+        ids = wl.indices[t]
+        rows, cnt = np.unique(ids, return_counts=True)
+        top = rows[np.argsort(-cnt, kind="stable")[:k_hot]].astype(np.int32)
+        top = np.concatenate([top, np.zeros(k_hot - top.size, np.int32)])      # a table of fewer rows than k_hot
+        lut = np.full(wl.rows[t], -1, np.int32)
+        lut[top[::-1]] = np.arange(k_hot - 1, -1, -1, dtype=np.int32)
+        out = np.empty_like(ids)
+        for s0 in range(0, ids.size, chunk):
+            c = ids[s0:s0 + chunk]
+            slot = lut[c]
+            hot = slot >= 0
+            out[s0:s0 + c.size] = np.concatenate([c[~hot], slot[hot]])
+            it_t.append(t), it_s.append(s0), it_c.append(c.size), it_h.append(int(hot.sum()))
+        n_hot_fetches += int(sum(it_h[-((ids.size + chunk - 1) // chunk):]))
+        streams.append(torch.from_numpy(out).cuda())
+        hots.append(torch.from_numpy(top).cuda())
+    n_items = len(it_t)
+    cost = ops.MultiTableBatch(tabs, streams, [torch.zeros(wl.n_bags, dtype=torch.int32, device="cuda")] * len(tabs)
+                               ).default_table_cost()
+    c = np.cumsum(cost[np.array(it_t)] * np.array(it_c))
+    c /= c[-1]
+    xs = [0] + [int(np.searchsorted(c, k / 8.0)) for k in range(1, 8)] + [n_items]
+    longest = max(xs[k + 1] - xs[k] for k in range(8))
+
+    class Args(C.Structure):
+        _fields_ = [("tables", C.c_void_p), ("item_table", C.c_void_p), ("item_start", C.c_void_p),
+                    ("item_count", C.c_void_p), ("item_hot", C.c_void_p), ("out", C.c_void_p),
+                    ("xcd_start", C.c_int32 * 9), ("store_every", C.c_int32), ("store_mode", C.c_int32),
+                    ("n_hot", C.c_int32), ("one", C.c_float)]
+    td = np.zeros((len(tabs), 3), np.int64)
+    for t in range(len(tabs)):
+        td[t] = (tabs[t].data_ptr(), streams[t].data_ptr(), hots[t].data_ptr())
+    d_td = torch.from_numpy(td).cuda()
+    d_t, d_s, d_c, d_h = (torch.tensor(a, dtype=torch.int32).cuda() for a in (it_t, it_s, it_c, it_h))
+    buf = torch.zeros((n_items * 16 * 64, 128), dtype=torch.float16, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    avg_len = wl.n_indices() / float(wl.n_bags * len(wl.rows))
+    every = max(8, int(round(avg_len / 8.0)) * 8)
+    res = {"hot_rows_per_table": k_hot, "share_of_fetches_served_by_lds": n_hot_fetches / float(wl.n_indices())}
+    for key, store_every, mode in (("gather_only_ms", 0, 1), ("gather_streaming_stores_ms", every, 2)):
+        a = Args(d_td.data_ptr(), d_t.data_ptr(), d_s.data_ptr(), d_c.data_ptr(), d_h.data_ptr(), buf.data_ptr(),
+                 (C.c_int32 * 9)(*xs), store_every, mode, k_hot, 1.0)
+
+        def fn():
+            rc = dll.fwdmi_mb_replay_hot(C.byref(a), longest, stream)
+            if rc:
+                raise RuntimeError("replay launch failed: hipError %d" % rc)
+        _, per = time_events(torch, fn, steps, 10)
+        res[key] = float(np.median(per))
+    return res
+
+
+def replay(torch, ops, workloads, ids_mode, order="stream", k_hot=0):
     """`--replay`: the product launch beside the bag-free replay of the same id stream (a table on stdout)."""
     wl = workloads.config4()
     rng = np.random.Generator(np.random.PCG64(1))
@@ -798,6 +866,14 @@ def replay(torch, ops, workloads, ids_mode, order="stream"):
                        ("gather + a 256 B result row every %d rows, stores confined to 4 MiB (never leave L2)" % e,
                         "gather_stores_within_4MiB_ms")):
         print("%-72s %8.4f ms" % (label, r[key]), flush=True)
+    if k_hot > 0:
+        del idx, off
+        h = replay_hot_times(torch, ops, wl, tabs, min(64, k_hot))
+        print("replay with the %d most frequent rows of every table in LDS (%.1f %% of the fetches):" %
+              (h["hot_rows_per_table"], 100.0 * h["share_of_fetches_served_by_lds"]))
+        print("%-72s %8.4f ms" % ("gather only (one result row per slot)", h["gather_only_ms"]), flush=True)
+        print("%-72s %8.4f ms" % ("gather + a 256 B result row every %d rows, non-temporal stores" % e,
+                                  h["gather_streaming_stores_ms"]), flush=True)
 
 
 def lru_sim(workloads, capacities=(8192, 12288, 16384, 32768)):
@@ -851,7 +927,7 @@ def main():
         sweep_layer_norm(torch, ops)
         return
     if args.replay:
-        replay(torch, ops, workloads, args.ids, args.order)
+        replay(torch, ops, workloads, args.ids, args.order, args.hot)
         return
 
     t0 = time.time()

@@ -228,3 +228,51 @@ def test_no_alloc_entry_point_under_graph_capture(oracle, n_tables):
         launch(other)                               # an eager call between the replays
         torch.cuda.synchronize()
         assert_bits_equal(host(other), want(ids, offs), "eager between replays %d" % seed)
+
+
+def test_no_alloc_calls_from_several_host_threads_on_one_stream(oracle):
+    """Four host threads issue calls of different table sets (each more tables than travel with a launch,
+    so all go through the shared descriptor buffer) on ONE stream.  A call's descriptor writes and its
+    launch are enqueued under one lock, so no thread's launch can read another's descriptors; every
+    output is checked against the oracle."""
+    import threading
+    rng = np.random.Generator(np.random.PCG64(404))
+    n_tables, dim, n_bags = lib.BAG_INLINE_TABLES + 3, 32, 300
+    stream = torch.cuda.Stream()
+    s = C.c_void_p(stream.cuda_stream)
+    sets = []
+    for k in range(4):
+        tables, ids, offs = make_batch(rng, [int(v) for v in rng.integers(5, 400, n_tables)], n_bags, dim, np.float32,
+                                       np.int32, 6)
+        d_tab, d_ids, d_off = [dev(t) for t in tables], [dev(i) for i in ids], [dev(o) for o in offs]
+        want = np.concatenate([oracle.embedding_bag(tables[t], ids[t], offs[t], 0)[0] for t in range(n_tables)], axis=1)
+        sets.append((d_tab, d_ids, d_off, descriptors(d_tab, d_ids, d_off, dim), want,
+                     float(sum(i.size for i in ids)) / (n_tables * n_bags)))
+    torch.cuda.synchronize()
+    rounds = 25
+    outs = [[torch.full((n_bags, n_tables * dim), -3.0, dtype=torch.float32, device="cuda") for _ in range(rounds)]
+            for _ in range(4)]
+    errors = []
+
+    def work(k):
+        try:
+            d_tab, d_ids, _, desc, _, avg = sets[k]
+            x = ops._ext(d_tab[0], d_ids[0], torch.float32, out_row_stride=n_tables * dim)
+            for r in range(rounds):
+                rc = lib.dll.fwdmi_embedding_bag_multi_noalloc(C.c_void_p(desc.ctypes.data), n_tables, n_bags,
+                                                               C.c_void_p(outs[k][r].data_ptr()), dim, 0, avg, C.byref(x), s)
+                if rc:
+                    raise RuntimeError("call failed: %d" % rc)
+        except Exception as e:       # pragma: no cover
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    stream.synchronize()
+    assert not errors, errors
+    for k in range(4):
+        for r in range(rounds):
+            assert_bits_equal(host(outs[k][r]), sets[k][4], "thread %d call %d" % (k, r))

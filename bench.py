@@ -1006,7 +1006,8 @@ def main():
                    "id_batches_are": ("step i works on batch i mod %d: fresh bag lengths and ids over the same tables, all "
                                       "resident in HBM before the timed region" % n_batches) if n_batches > 1 else
                                      "every step replays the same batch",
-                   "total_ids": wl.n_indices(), "table_bytes": int(sum(t.numel() * 2 for t in tabs))},
+                   "total_ids": wl.n_indices(), "table_bytes": int(sum(t.numel() * 2 for t in tabs)),
+                   "device": dict(zip(("compute_units", "xcds"), ops.device_topology()))},
         "roofline": {
             "bound": "hbm",
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",

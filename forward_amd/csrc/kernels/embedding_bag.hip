@@ -931,6 +931,16 @@ int fwdmi_embedding_bag_multi_noalloc(const fwdmi_bag_table* tables_host, int32_
                              static_cast<hipStream_t>(stream));
 }
 
+int fwdmi_bag_device_topology(int32_t* cus, int32_t* xcds) {
+  fwdmi::clear_error();
+  if (!cus || !xcds) return fwdmi::set_error(FWDMI_ERR_BAD_ARG, "device topology: null argument");
+  fwdmi::BagTopology topo{0, 1};
+  if (const int rc = fwdmi::device_topology(&topo)) return rc;
+  *cus = topo.cus;
+  *xcds = topo.xcds;
+  return FWDMI_OK;
+}
+
 // Measured on the 26-table configuration (tables of 0.25 MB .. 2.5 GB): per-bag cost ratios
 // between 1.3 and 1.6 for HBM-resident against L2-resident tables balance the eight XCDs best.
 int fwdmi_bag_table_cost(const int64_t* table_bytes, int32_t n_tables, float* cost) {

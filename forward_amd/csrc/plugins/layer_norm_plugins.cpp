@@ -295,6 +295,11 @@ EmbLayerNormPluginDynamic::EmbLayerNormPluginDynamic(std::string name, DataType 
       batch_major_(batch_major), t_(std::move(tables)) {
   std::vector<float> all(t_.beta);
   all.insert(all.end(), t_.gamma.begin(), t_.gamma.end());
+  if (t_.fused_skip) {
+    all.insert(all.end(), t_.beta2.begin(), t_.beta2.end());
+    all.insert(all.end(), t_.gamma2.begin(), t_.gamma2.end());
+    all.insert(all.end(), t_.bias2.begin(), t_.bias2.end());
+  }
   params_ = make_blob_f32(all);
 }
 
@@ -310,12 +315,24 @@ IPluginV2DynamicExt* EmbLayerNormPluginDynamic::clone() const noexcept {
 // Inputs are three [S, B] id tensors (trt_bert_creator.h:64-71).  Output 0 is the embedding
 // consumed as [S, B, H, 1, 1] (plugins/common/plugin_common.h:39-41); output 1 is the mask index,
 // one int per batch row in the unfused layout (plugin_common.h:63,77-94).  With the optional
-// `batch_major` field the ids are [B, S] and output 0 is [B, S, H, 1, 1].
+// `batch_major` field the ids are [B, S] and output 0 is [B, S, H, 1, 1].  A plugin that also stands for
+// the SkipLayerNorm behind it (fields skip_beta / skip_gamma, trt_bert_creator.h:199-239) takes that
+// layer's second input, the residual, as its fourth: shaped like output 0 ([.., .., H] or [.., .., H, 1, 1]).
 Dims EmbLayerNormPluginDynamic::getOutputDimensions(int outputIndex, const Dims* inputs, int nbInputs) noexcept {
   clear_error();
-  if (!inputs || nbInputs != 3 || outputIndex < 0 || outputIndex > 1) {
-    set_error(FWDMI_ERR_BAD_ARG, "EmbLayerNorm: output %d with %d inputs", outputIndex, nbInputs);
+  if (!inputs || nbInputs != nb_inputs() || outputIndex < 0 || outputIndex > 1) {
+    set_error(FWDMI_ERR_BAD_ARG, "EmbLayerNorm: output %d with %d inputs (the plugin takes %d)", outputIndex, nbInputs,
+              nb_inputs());
     return error_dims();
+  }
+  if (t_.fused_skip) {
+    const Dims& r = inputs[3];
+    bool ok = (r.nbDims == 3 || r.nbDims == 5) && r.d[0] == inputs[0].d[0] && r.d[1] == inputs[0].d[1] && r.d[2] == ld_;
+    for (int i = 3; ok && i < r.nbDims; ++i) ok = r.d[i] == 1;
+    if (!ok) {
+      set_error(FWDMI_ERR_BAD_ARG, "EmbLayerNorm: the residual input must be shaped like the embedding output");
+      return error_dims();
+    }
   }
   for (int i = 0; i < 3; ++i)
     if (inputs[i].nbDims != 2 || inputs[i].d[0] != inputs[0].d[0] || inputs[i].d[1] != inputs[0].d[1]) {
@@ -340,17 +357,17 @@ Dims EmbLayerNormPluginDynamic::getOutputDimensions(int outputIndex, const Dims*
 
 bool EmbLayerNormPluginDynamic::supportsFormatCombination(int pos, const PluginTensorDesc* inOut, int nbInputs,
                                                           int nbOutputs) noexcept {
-  if (!inOut || nbInputs != 3 || nbOutputs != 2 || pos < 0 || pos >= 5) return false;
+  if (!inOut || nbInputs != nb_inputs() || nbOutputs != 2 || pos < 0 || pos >= nbInputs + 2) return false;
   const PluginTensorDesc& d = inOut[pos];
   if (d.format != FWDMI_FORMAT_LINEAR) return false;
-  if (pos == 3) return d.type == (int32_t)type_;
+  if (pos == nbInputs || (t_.fused_skip && pos == 3)) return d.type == (int32_t)type_;  // output 0, the residual
   return d.type == FWDMI_I32;
 }
 
 int EmbLayerNormPluginDynamic::configurePlugin(const DynamicPluginTensorDesc* in, int nbInputs,
                                                const DynamicPluginTensorDesc*, int nbOutputs) noexcept {
   clear_error();
-  if (!in || nbInputs != 3 || nbOutputs != 2)
+  if (!in || nbInputs != nb_inputs() || nbOutputs != 2)
     return set_error(FWDMI_ERR_BAD_ARG, "EmbLayerNorm::configurePlugin: %d inputs, %d outputs", nbInputs, nbOutputs);
   if (configured_) return FWDMI_OK;
   void* p = nullptr;
@@ -395,6 +412,16 @@ int EmbLayerNormPluginDynamic::enqueue(const PluginTensorDesc* inputDesc, const 
   const int S = inputDesc[0].dims.d[batch_major_ ? 1 : SDIM], B = inputDesc[0].dims.d[batch_major_ ? 0 : BDIM];
   fwdmi_emb_ext ext{};
   ext.batch_major = batch_major_ ? 1 : 0;
+  if (t_.fused_skip) {
+    if (inputDesc[3].type != (int32_t)type_)
+      return set_error(FWDMI_ERR_UNSUPPORTED, "EmbLayerNorm: the residual input has type %d, the output %d",
+                       inputDesc[3].type, (int32_t)type_);
+    ext.skip = inputs[3];
+    ext.beta2 = d_params_ + 2 * (size_t)ld_;
+    ext.gamma2 = d_params_ + 3 * (size_t)ld_;
+    ext.bias2 = t_.bias2.empty() ? nullptr : d_params_ + 4 * (size_t)ld_;
+    ext.eps2 = t_.eps2;
+  }
   return fwdmi_emb_layer_norm_ex(hipStream, S, B, ld_, static_cast<const int32_t*>(inputs[0]),
                                  static_cast<const int32_t*>(inputs[1]), static_cast<const int32_t*>(inputs[2]),
                                  d_params_, d_params_ + ld_, d_word_, d_pos_, d_tok_, t_.word_count, t_.pos_count,
@@ -425,10 +452,14 @@ void EmbLayerNormPluginDynamic::terminate() noexcept {
 // Own layout (the NVIDIA plugin's bytes are not part of the reference tree):
 //   int type | int mha_type | int ld | int word_count | int pos_count | int tok_count | float eps |
 //   beta f32[ld] | gamma f32[ld] | word[word_count*ld] | pos[pos_count*ld] | tok[tok_count*ld]
-// followed, only for a batch-major plugin, by int batch_major(4).
+// followed, only for a batch-major plugin or one that also stands for the SkipLayerNorm behind it, by
+// int batch_major, and for the latter by int 1 | float eps2 | int has_bias2 | beta2 f32[ld] | gamma2 f32[ld] [| bias2 f32[ld]].
 size_t EmbLayerNormPluginDynamic::getSerializationSize() const noexcept {
-  return 6 * sizeof(int32_t) + sizeof(float) + 2 * (size_t)ld_ * sizeof(float) + t_.word->size() +
-         t_.pos->size() + t_.tok->size() + (batch_major_ ? sizeof(int32_t) : 0);
+  size_t n = 6 * sizeof(int32_t) + sizeof(float) + 2 * (size_t)ld_ * sizeof(float) + t_.word->size() +
+             t_.pos->size() + t_.tok->size() + ((batch_major_ || t_.fused_skip) ? sizeof(int32_t) : 0);
+  if (t_.fused_skip)
+    n += 2 * sizeof(int32_t) + sizeof(float) + (2 + (t_.bias2.empty() ? 0 : 1)) * (size_t)ld_ * sizeof(float);
+  return n;
 }
 
 void EmbLayerNormPluginDynamic::serialize(void* buffer) const noexcept {
@@ -445,7 +476,15 @@ void EmbLayerNormPluginDynamic::serialize(void* buffer) const noexcept {
   w.bytes(t_.word->data(), t_.word->size());
   w.bytes(t_.pos->data(), t_.pos->size());
   w.bytes(t_.tok->data(), t_.tok->size());
-  if (batch_major_) w.pod<int32_t>(1);
+  if (batch_major_ || t_.fused_skip) w.pod<int32_t>(batch_major_ ? 1 : 0);
+  if (t_.fused_skip) {
+    w.pod<int32_t>(1);
+    w.pod<float>(t_.eps2);
+    w.pod<int32_t>(t_.bias2.empty() ? 0 : 1);
+    w.bytes(t_.beta2.data(), t_.beta2.size() * 4);
+    w.bytes(t_.gamma2.data(), t_.gamma2.size() * 4);
+    w.bytes(t_.bias2.data(), t_.bias2.size() * 4);
+  }
 }
 
 EmbLayerNormPluginDynamic* EmbLayerNormPluginDynamic::deserialize(const std::string& name, const void* data,
@@ -493,6 +532,25 @@ EmbLayerNormPluginDynamic* EmbLayerNormPluginDynamic::deserialize(const std::str
   t.tok = read_table(t.tok_count);
   int32_t batch_major = 0;
   if (r.left() >= sizeof(int32_t)) r.pod(&batch_major);
+  if (r.left() > 0) {  // the SkipLayerNorm the plugin also stands for
+    int32_t fused = 0, has_bias = 0;
+    r.pod(&fused);
+    r.pod(&t.eps2);
+    r.pod(&has_bias);
+    if (!r.ok() || fused != 1 || (has_bias != 0 && has_bias != 1) || r.left() != (size_t)(2 + has_bias) * ld * 4) {
+      set_error(FWDMI_ERR_TRUNCATED, "EmbLayerNorm: serialized second stage truncated or malformed");
+      return nullptr;
+    }
+    t.fused_skip = true;
+    t.beta2.resize(ld);
+    t.gamma2.resize(ld);
+    r.bytes(t.beta2.data(), (size_t)ld * 4);
+    r.bytes(t.gamma2.data(), (size_t)ld * 4);
+    if (has_bias) {
+      t.bias2.resize(ld);
+      r.bytes(t.bias2.data(), (size_t)ld * 4);
+    }
+  }
   if (!r.ok()) {
     set_error(FWDMI_ERR_TRUNCATED, "EmbLayerNorm: serialized tables truncated");
     return nullptr;
@@ -515,6 +573,11 @@ EmbLayerNormPluginDynamicCreator::EmbLayerNormPluginDynamicCreator() {
   declare("mha_type_id", PluginFieldType::kINT32);
   declare("eps", PluginFieldType::kFLOAT32);
   declare("batch_major", PluginFieldType::kINT32);
+  // the SkipLayerNorm behind the embedding (its own fields are beta / gamma / bias, trt_bert_creator.h:219-229)
+  declare("skip_beta", PluginFieldType::kFLOAT32);
+  declare("skip_gamma", PluginFieldType::kFLOAT32);
+  declare("skip_bias", PluginFieldType::kFLOAT32);
+  declare("skip_eps", PluginFieldType::kFLOAT32);
 }
 
 IPluginV2DynamicExt* EmbLayerNormPluginDynamicCreator::createPlugin(const char* name,
@@ -524,9 +587,9 @@ IPluginV2DynamicExt* EmbLayerNormPluginDynamicCreator::createPlugin(const char* 
     set_error(FWDMI_ERR_BAD_ARG, "EmbLayerNorm: null field collection");
     return nullptr;
   }
-  std::vector<float> beta, gamma, word, tok, pos;
+  std::vector<float> beta, gamma, word, tok, pos, beta2, gamma2, bias2;
   int output_fp16 = 0, mha_type = 0, batch_major = 0;
-  float eps = 0.0f;
+  float eps = 0.0f, eps2 = 0.0f;
   for (int i = 0; i < fc->nbFields; ++i) {
     const PluginField& f = fc->fields[i];
     const std::string n = f.name ? f.name : "";
@@ -540,6 +603,10 @@ IPluginV2DynamicExt* EmbLayerNormPluginDynamicCreator::createPlugin(const char* 
     else if (n == "output_fp16") ok = f.data && f.type == FWDMI_FIELD_I32, output_fp16 = ok ? *static_cast<const int*>(f.data) : 0;
     else if (n == "mha_type_id") ok = f.data && f.type == FWDMI_FIELD_I32, mha_type = ok ? *static_cast<const int*>(f.data) : 0;
     else if (n == "eps") ok = f.data && f.type == FWDMI_FIELD_F32, eps = ok ? *static_cast<const float*>(f.data) : 0.0f;
+    else if (n == "skip_beta") ok = field_to_f32(f, &beta2);
+    else if (n == "skip_gamma") ok = field_to_f32(f, &gamma2);
+    else if (n == "skip_bias") ok = field_to_f32(f, &bias2);
+    else if (n == "skip_eps") ok = f.data && f.type == FWDMI_FIELD_F32, eps2 = ok ? *static_cast<const float*>(f.data) : 0.0f;
     if (!ok) {
       set_error(FWDMI_ERR_BAD_ARG, "EmbLayerNorm: field '%s' has the wrong type or no data", n.c_str());
       return nullptr;
@@ -552,8 +619,18 @@ IPluginV2DynamicExt* EmbLayerNormPluginDynamicCreator::createPlugin(const char* 
               beta.size(), gamma.size(), word.size(), pos.size(), tok.size());
     return nullptr;
   }
+  const bool fused = !beta2.empty() || !gamma2.empty() || !bias2.empty();
+  if (fused && (beta2.size() != ld || gamma2.size() != ld || (!bias2.empty() && bias2.size() != ld))) {
+    set_error(FWDMI_ERR_BAD_ARG, "EmbLayerNorm: skip_beta / skip_gamma (/ skip_bias) must hold %zu values each", ld);
+    return nullptr;
+  }
   const DataType type = output_fp16 ? DataType::kHALF : DataType::kFLOAT;
   EmbLayerNormPluginDynamic::Tables t;
+  t.fused_skip = fused;
+  t.beta2 = std::move(beta2);
+  t.gamma2 = std::move(gamma2);
+  t.bias2 = std::move(bias2);
+  t.eps2 = eps2;
   t.word_count = (int)(word.size() / ld);
   t.pos_count = (int)(pos.size() / ld);
   t.tok_count = (int)(tok.size() / ld);

@@ -108,6 +108,11 @@ class EmbLayerNormPluginDynamic final : public IPluginV2DynamicExt {
     std::vector<float> beta, gamma;                // [ld] fp32
     std::shared_ptr<HostDeviceBlob> word, pos, tok;  // rows in the output type
     int word_count = 0, pos_count = 0, tok_count = 0;
+    // The SkipLayerNorm that consumes the embedding, when the plugin stands for both layers: a fourth
+    // input (the residual, shaped like output 0) and output 0 = LN2(embedding + residual (+ bias2)).
+    bool fused_skip = false;
+    std::vector<float> beta2, gamma2, bias2;  // [ld] fp32; bias2 may be empty
+    float eps2 = 0.0f;
   };
   EmbLayerNormPluginDynamic(std::string name, DataType type, DataType mha_type, int ld, Tables tables, float eps,
                             bool batch_major = false);
@@ -144,7 +149,8 @@ class EmbLayerNormPluginDynamic final : public IPluginV2DynamicExt {
   float eps_;
   bool batch_major_;  // ids are [B, S] and the output [B, S, H, 1, 1] (no transposes around the plugin)
   Tables t_;
-  std::shared_ptr<HostDeviceBlob> params_;  // beta | gamma fp32
+  std::shared_ptr<HostDeviceBlob> params_;  // beta | gamma [| beta2 | gamma2 [| bias2]] fp32
+  int nb_inputs() const { return t_.fused_skip ? 4 : 3; }
   float* d_params_ = nullptr;
   void *d_word_ = nullptr, *d_pos_ = nullptr, *d_tok_ = nullptr;
   int32_t* d_oob_ = nullptr;

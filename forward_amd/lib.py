@@ -89,6 +89,7 @@ SIGNATURES = {
     "fwdmi_embedding_bag_fixed": (C.c_int, [_vp, _vp, _i64, _i64, _vp, _i64, _i32, _i64, _i32, C.POINTER(BagExt), _vp]),
     "fwdmi_gather": (C.c_int, [_vp, _vp, _i64, _i64, _vp, _i64, _i32, _i64, C.POINTER(BagExt), _vp]),
     "fwdmi_bag_table_cost": (C.c_int, [_vp, _i32, _vp]),
+    "fwdmi_bag_device_topology": (C.c_int, [C.POINTER(_i32), C.POINTER(_i32)]),
     "fwdmi_bag_tables_fill": (C.c_int, [_vp, _i32, _vp, _vp]),
     "fwdmi_embedding_bag_multi": (C.c_int, [_vp, _i32, _i64, _vp, _i32, _i32, C.c_double, C.POINTER(BagExt), _vp]),
     "fwdmi_embedding_bag_multi_host": (C.c_int, [_vp, _i32, _vp, _i64, _vp, _i32, _i32, C.c_double, C.POINTER(BagExt),

@@ -136,6 +136,13 @@ def gather(table, indices, data_offset=0, out_dtype=None, oob_flag=None, stream=
     return out
 
 
+def device_topology():
+    """``(compute units, XCDs)`` of the current device as the bag launches see them."""
+    cus, xcds = C.c_int32(0), C.c_int32(0)
+    lib.check(lib.dll.fwdmi_bag_device_topology(C.byref(cus), C.byref(xcds)))
+    return int(cus.value), int(xcds.value)
+
+
 class MultiTableBatch:
     """Device-resident descriptor array for ``fwdmi_embedding_bag_multi``.
 

@@ -239,6 +239,14 @@ int fwdmi_bag_tables_fill(const fwdmi_bag_table* tables_host, int32_t n_tables, 
 int fwdmi_bag_table_cost(const int64_t* table_bytes, int32_t n_tables, float* cost);
 
 /*
+ * What the bag launches know of the current device, as the runtime reports it: compute units and
+ * XCDs (accelerator dies, one L2 each; 1 when the device is one die or the runtime does not say).
+ * Run sizes follow the CU count; FWDMI_BAG_XCD_TABLE_AFFINITY is honoured with 2 .. 8 XCDs and is
+ * the plain table-major order otherwise.  (No counterpart in the reference.)
+ */
+int fwdmi_bag_device_topology(int32_t* cus, int32_t* xcds);
+
+/*
  * out = gamma * (x - mean) * rsqrt(var + eps) + beta,  x = input (+ bias), per row of ld.
  * n = total elements (rows = n / ld).  gamma/beta/bias: device fp32 [ld]; bias may be NULL.
  * dtype: FWDMI_F32 | FWDMI_F16 for input and output.  The reference has no eps (pass 0).

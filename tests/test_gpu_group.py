@@ -356,3 +356,13 @@ def test_host_descriptor_entry_point_limits(oracle):
         desc[2, 2] = 0
     rc, got, *_ = call(3, None, no_offsets)
     assert rc == lib.ERR_BAD_ARG and "offsets" in lib.last_error() and (got == 9.0).all()
+
+
+def test_device_topology_is_reported():
+    """The bag launches size themselves from what the runtime says of the device; the same figures are
+    available to the caller (and end up in bench.py's JSON)."""
+    from forward_amd import ops
+    cus, xcds = ops.device_topology()
+    assert cus > 0 and 1 <= xcds <= cus
+    props = torch.cuda.get_device_properties(0)
+    assert cus == props.multi_processor_count

@@ -224,6 +224,53 @@ def test_plugins_config5_chain(oracle):
         skip.configurePlugin([((64, 4, 1024), lib.F32)] * 2, [((64, 4, 1024), lib.F32)])
 
 
+@pytest.mark.parametrize("batch_major", [False, True])
+def test_one_plugin_for_embedding_and_skip_layer_norm_equals_the_two_plugins(oracle, batch_major):
+    """CustomEmbLayerNormPluginDynamic with the skip_* fields stands for the embedding plugin and the
+    SkipLayerNorm plugin behind it: one enqueue, bit-identical to the chain of the two, in both id layouts,
+    also after serialize -> deserialize; against the oracle within the fp16 bar."""
+    wl = workloads.config5(variant=2, batch=3, seq=80)
+    up = lambda a: a.astype(np.float32)
+    S, B, H = 80, 3, 1024
+    lay = (lambda a: np.ascontiguousarray(np.swapaxes(a, 0, 1))) if batch_major else (lambda a: a)
+    ids, seg, msk = (dev(lay(a)) for a in (wl.input_ids, wl.segment_ids, wl.input_mask))
+    res = dev(lay(wl.skip).reshape(tuple(lay(wl.input_ids).shape) + (H, 1, 1)))
+    emb_f = [F("bert_embeddings_layernorm_beta", up(wl.beta)), F("bert_embeddings_layernorm_gamma", up(wl.gamma)),
+             F("bert_embeddings_word_embeddings", up(wl.word)), F("bert_embeddings_token_type_embeddings", up(wl.tok)),
+             F("bert_embeddings_position_embeddings", up(wl.pos)), F("output_fp16", 1), F("mha_type_id", lib.F16),
+             F("eps", np.array([wl.eps], np.float32)), F("batch_major", int(batch_major))]
+    ce = REG.getPluginCreator("CustomEmbLayerNormPluginDynamic", "1")
+    cs = REG.getPluginCreator("CustomSkipLayerNormPluginDynamic", "1")
+    e, midx = ce.createPlugin("embeddings", emb_f)(ids, seg, msk)
+    want = cs.createPlugin("skip_ln", [F("beta", up(wl.skip_beta)), F("gamma", up(wl.skip_gamma)), F("ld", H),
+                                       F("type_id", lib.F16), F("bias", up(wl.skip_bias)),
+                                       F("eps", np.array([wl.eps], np.float32))])(e, res)
+    both = ce.createPlugin("embeddings+skip", emb_f + [
+        F("skip_beta", up(wl.skip_beta)), F("skip_gamma", up(wl.skip_gamma)), F("skip_bias", up(wl.skip_bias)),
+        F("skip_eps", np.array([wl.eps], np.float32))])
+    got, gmidx = both(ids, seg, msk, res)
+    assert tuple(got.shape) == tuple(e.shape)
+    np.testing.assert_array_equal(host(got).view(np.uint16), host(want).view(np.uint16))
+    np.testing.assert_array_equal(host(gmidx), host(midx))
+    got2, _ = ce.deserializePlugin("embeddings+skip", both.serialize())(ids, seg, msk, res)
+    np.testing.assert_array_equal(host(got2).view(np.uint16), host(want).view(np.uint16))
+    wemb, wmidx, _ = oracle.emb_layer_norm(wl.input_ids, wl.segment_ids, wl.input_mask, wl.word, wl.pos, wl.tok,
+                                           wl.gamma, wl.beta, eps=wl.eps)
+    wout = oracle.skip_layer_norm(wemb, wl.skip_gamma, wl.skip_beta, skip=wl.skip, bias=wl.skip_bias, eps=wl.eps)
+    g = host(got).reshape(tuple(lay(wl.input_ids).shape) + (H,))
+    assert_close(np.swapaxes(g, 0, 1) if batch_major else g, wout, np.float16)
+    np.testing.assert_array_equal(host(gmidx).reshape(-1), wmidx)
+    # without a bias, and a residual of the wrong type is refused
+    nob = ce.createPlugin("embeddings+skip", emb_f + [F("skip_beta", up(wl.skip_beta)), F("skip_gamma", up(wl.skip_gamma)),
+                                                      F("skip_eps", np.array([wl.eps], np.float32))])
+    got3, _ = nob(ids, seg, msk, res)
+    want3 = cs.createPlugin("skip_ln", [F("beta", up(wl.skip_beta)), F("gamma", up(wl.skip_gamma)), F("ld", H),
+                                        F("type_id", lib.F16), F("eps", np.array([wl.eps], np.float32))])(e, res)
+    np.testing.assert_array_equal(host(got3).view(np.uint16), host(want3).view(np.uint16))
+    with pytest.raises(lib.FwdmiError):
+        nob(ids, seg, msk, res.float())
+
+
 def test_launches_can_be_captured_in_a_hip_graph(oracle):
     """enqueue allocates nothing and never synchronises, so a chain of launches can be captured
     once and replayed; every replay (with eager work in between) must equal the eager result."""

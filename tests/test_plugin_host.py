@@ -280,6 +280,49 @@ def emb_fields(rng, ld=16, vocab=40, pos=12, fp16=0):
             F("bert_embeddings_position_embeddings", r(pos, ld)), F("output_fp16", fp16), F("mha_type_id", fp16)]
 
 
+def test_emb_layer_norm_plugin_that_also_stands_for_the_skip_layer_norm_host_contract():
+    """Optional fields skip_beta / skip_gamma (/ skip_bias, skip_eps): the plugin takes the SkipLayerNorm's
+    second input (the residual) as its fourth and stands for both layers (trt_bert_creator.h:113-155,199-239)."""
+    rng = np.random.default_rng(5)
+    c = REG.getPluginCreator("CustomEmbLayerNormPluginDynamic", "1")
+    r = lambda n: rng.standard_normal(n).astype(np.float32)
+    base = emb_fields(rng, fp16=1)
+    for with_bias in (False, True):
+        extra = [F("skip_beta", r(16)), F("skip_gamma", r(16)), F("skip_eps", np.array([1e-6], np.float32))]
+        if with_bias:
+            extra.append(F("skip_bias", r(16)))
+        p = c.createPlugin("embeddings", base + extra)
+        ins = [(12, 4)] * 3 + [(12, 4, 16, 1, 1)]
+        assert p.getNbOutputs() == 2
+        assert p.getOutputDimensions(0, ins) == [12, 4, 16, 1, 1] and p.getOutputDimensions(1, ins) == [4, 1]
+        assert p.getOutputDimensions(0, ins[:3] + [(12, 4, 16)]) == [12, 4, 16, 1, 1]
+        with pytest.raises(lib.FwdmiError, match="takes 4"):
+            p.getOutputDimensions(0, ins[:3])
+        with pytest.raises(lib.FwdmiError, match="residual"):
+            p.getOutputDimensions(0, ins[:3] + [(12, 4, 17, 1, 1)])
+        io = [((12, 4), lib.I32)] * 3 + [((12, 4, 16, 1, 1), lib.F16), ((12, 4, 16, 1, 1), lib.F16), ((4, 1), lib.I32)]
+        assert all(p.supportsFormatCombination(i, io, 4, 2) for i in range(6))
+        assert not p.supportsFormatCombination(3, io[:3] + [((12, 4, 16, 1, 1), lib.F32)] + io[4:], 4, 2)
+        assert not p.supportsFormatCombination(0, io[:3] + io[4:], 3, 2)               # the plain plugin's shape
+        blob = p.serialize()
+        plain = c.createPlugin("embeddings", base).serialize()
+        n2 = (3 if with_bias else 2) * 16 * 4
+        assert len(blob) == p.getSerializationSize() == len(plain) + 4 + 12 + n2
+        assert blob[:len(plain)] == plain                                                # the plain plugin's bytes first
+        assert struct.unpack("<iifi", blob[len(plain):len(plain) + 16]) == (0, 1, np.float32(1e-6), int(with_bias))
+        assert blob[len(plain) + 16:len(plain) + 16 + 64] == extra[0].array.tobytes()
+        q = c.deserializePlugin("e", blob)
+        assert q.serialize() == blob and p.clone().serialize() == blob
+        assert q.getOutputDimensions(0, ins) == [12, 4, 16, 1, 1]
+        for cut in (1, 5, 64, n2 + 3):
+            with pytest.raises(lib.FwdmiError):
+                c.deserializePlugin("e", blob[:-cut])
+    with pytest.raises(lib.FwdmiError, match="skip_beta"):
+        c.createPlugin("x", base + [F("skip_beta", r(16))])                              # gamma missing
+    with pytest.raises(lib.FwdmiError, match="skip_beta"):
+        c.createPlugin("x", base + [F("skip_beta", r(16)), F("skip_gamma", r(15))])
+
+
 def test_emb_layer_norm_plugin_host_contract():
     rng = np.random.default_rng(3)
     c = REG.getPluginCreator("CustomEmbLayerNormPluginDynamic", "1")

@@ -55,24 +55,48 @@ constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 // ranges come in with 16-byte loads (a load instruction occupies the CU's memory pipeline for the
 // same time whatever its width); the elements before the first 16-byte boundary and behind the
 // last one go one by one, so nothing outside the range is read.  `first` is aligned to its type.
+// All loads of a lane's share (up to four vectors, the two ends) are issued before the first of
+// them is used: the workgroup waits for memory once, not once per vector and once per end (a run of
+// 1830 ids is two vectors for most lanes, and most runs start and end off a 16-byte boundary).
 template <typename T, typename Put>
 __device__ __forceinline__ void stream_in(const T FWDMI_GLOBAL* first, int n, int tid, int lanes, Put put) {
   constexpr int kPer = 16 / (int)sizeof(T);
-  if (n < 2 * lanes) {  // uniform over the workgroup: too short for the split to pay
-    for (int i = tid; i < n; i += lanes) put(i, first[i]);
+  constexpr int kAhead = 4;  // vectors a lane has in flight
+  if (n < 2 * lanes) {  // uniform over the workgroup: too short for the split to pay; two elements per lane at most
+    const int i0 = tid, i1 = tid + lanes;
+    T a{}, b{};
+    if (i0 < n) a = first[i0];
+    if (i1 < n) b = first[i1];
+    if (i0 < n) put(i0, a);
+    if (i1 < n) put(i1, b);
     return;
   }
   const int misalign = (int)((reinterpret_cast<uintptr_t>(first) & 15) / sizeof(T));
   const int head = (kPer - misalign) & (kPer - 1);
   const int n_vec = (n - head) / kPer;
   const int body_end = head + n_vec * kPer;
-  for (int v = tid; v < n_vec; v += lanes) {
-    const Pack<T, kPer> p = gload<T, kPer>(first + head + v * kPer);
+  const bool has_head = tid < head, has_tail = body_end + tid < n;
+  T at_head{}, at_tail{};
+  if (has_head) at_head = first[tid];
+  if (has_tail) at_tail = first[body_end + tid];
+  for (int v0 = tid; v0 < n_vec; v0 += kAhead * lanes) {
+    Pack<T, kPer> p[kAhead];
 #pragma unroll
-    for (int e = 0; e < kPer; ++e) put(head + v * kPer + e, p.v[e]);
+    for (int k = 0; k < kAhead; ++k) {
+      const int v = v0 + k * lanes;
+      if (v < n_vec) p[k] = gload<T, kPer>(first + head + v * kPer);
+    }
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+      const int v = v0 + k * lanes;
+      if (v < n_vec) {
+#pragma unroll
+        for (int e = 0; e < kPer; ++e) put(head + v * kPer + e, p[k].v[e]);
+      }
+    }
   }
-  if (tid < head) put(tid, first[tid]);
-  if (body_end + tid < n) put(body_end + tid, first[body_end + tid]);
+  if (has_head) put(tid, at_head);
+  if (has_tail) put(body_end + tid, at_tail);
 }
 
 // EXT: the launch may use what only some multi-table launches need (runs sized per table, descriptors

@@ -62,7 +62,8 @@ struct BagLaunch {
   int32_t n_slices;
   int32_t bags_per_wg;
   int32_t wgs_per_table;
-  int32_t vec_store;  // 0: element stores; 1: 16-byte stores; 2: 16-byte stores with the non-temporal hint
+  int32_t vec_store;  // 0: element stores; 1: 16-byte stores; 2: 16-byte stores with the non-temporal hint;
+                      // 3: as 2 for 32 bytes of results per lane, halves traded between lanes first
   float one;  // 1.0f
   int32_t xcd_affinity;  // != 0: die x works through work items [xcd_start[x], xcd_start[x+1]); then the number of dies
   int32_t xcd_start[kMaxXcds + 1];

@@ -603,7 +603,30 @@ __global__ __launch_bounds__(kWG) FWDMI_BAG_OCCUPANCY void bag_reduce_kernel(con
           Pack<float, VEC> r;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) r.v[e] = acc[e];
-          if (VEC > 1 && L.vec_store == 2) {
+          if (VEC == 8 && L.vec_store == 3) {
+            // Eight fp32 results per lane are 32 bytes: stored as they lie, each of the two 16-byte
+            // store instructions would write every other 16 bytes of the slot's G * 32.  The lanes
+            // trade halves first (lane g takes what lane g/2, then lane G/2 + g/2, holds), so that
+            // each instruction writes one contiguous half.  Every lane of the slot is here: the
+            // plan asks for this form only when all column slices are full.
+            if constexpr (VEC == 8) {
+              const int lane = threadIdx.x & 63;
+              const int from0 = ((lane & ~(G - 1)) + (gl >> 1)) << 2, from1 = from0 + (G << 1);
+              const bool upper = gl & 1;
+              Pack<float, 4> h0, h1;
+#pragma unroll
+              for (int k = 0; k < 4; ++k) {
+                const int lo = __float_as_int(r.v[k]), hi = __float_as_int(r.v[4 + k]);
+                const int lo0 = __builtin_amdgcn_ds_bpermute(from0, lo), hi0 = __builtin_amdgcn_ds_bpermute(from0, hi);
+                const int lo1 = __builtin_amdgcn_ds_bpermute(from1, lo), hi1 = __builtin_amdgcn_ds_bpermute(from1, hi);
+                h0.v[k] = __int_as_float(upper ? hi0 : lo0);
+                h1.v[k] = __int_as_float(upper ? hi1 : lo1);
+              }
+              float FWDMI_GLOBAL* const slice = op - gl * VEC;  // the slot's first column of this slice
+              gstore_stream<float, 4>(slice + gl * 4, h0);
+              gstore_stream<float, 4>(slice + G * 4 + gl * 4, h1);
+            }
+          } else if (VEC > 1 && L.vec_store == 2) {
             if constexpr (VEC > 1) gstore_stream<float, VEC>(op, r);
           } else {
             gstore<float, VEC>(op, r);

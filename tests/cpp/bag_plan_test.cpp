@@ -59,6 +59,15 @@ static void walk(const Case& c, const BagPlan& P) {
   EXPECT(L.bags_per_wg >= 1 && L.bags_per_wg <= kMaxBagsPerWG, "%s: bags_per_wg %d", c.name.c_str(), L.bags_per_wg);
   EXPECT(L.idx_cap >= 1 && (size_t)L.idx_cap * 4 <= (size_t)kIdxBytes, "%s: idx_cap %d", c.name.c_str(), L.idx_cap);
   EXPECT(L.n_bags == c.n_bags, "%s: n_bags", c.name.c_str());
+  const int per_lane = P.vec ? (P.f16 ? 8 : 4) : 1;  // elements of a table row a lane holds
+  EXPECT(L.vec_store >= 0 && L.vec_store <= 3 && (per_lane > 1 || L.vec_store == 0), "%s: vec_store %d with %d elements per lane",
+         c.name.c_str(), L.vec_store, per_lane);
+  if (L.vec_store == 3) {  // halves traded between the lanes of a slot: every lane of every slice must hold results
+    const int g = 1 << L.log2_g;
+    EXPECT(per_lane == 8 && !L.out_f16 && g >= 2 && c.dim == L.n_slices * g * 8,
+           "%s: traded halves with %d elements per lane, fp16 results %d, slots of %d lanes, %d slices for %d columns",
+           c.name.c_str(), per_lane, (int)L.out_f16, g, L.n_slices, c.dim);
+  }
   if (L.var_runs) {
     EXPECT(P.ext, "%s: per-table run sizes need the extended kernel", c.name.c_str());
     EXPECT(L.run_start[0] == 0 && L.run_start[n_tables] == L.total_wgs, "%s: run_start ends", c.name.c_str());

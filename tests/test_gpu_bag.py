@@ -537,6 +537,34 @@ def test_results_large_enough_for_streaming_stores(oracle, tdt, odt):
     assert_bits_equal(host(s2), want2, "square sum of the two-output form")
 
 
+@pytest.mark.parametrize("dim", [8, 16, 32, 64, 72, 200, 256, 512, 1024, 2048])
+def test_fp32_results_of_fp16_tables_at_every_slot_width(oracle, dim):
+    """Eight fp32 results per lane leave in two 16-byte stores; where every column slice is full
+    (row widths of 2 .. 64 lanes, and 2048 columns in four slices) the lanes of a slot trade
+    halves first so that each store writes contiguous bytes, elsewhere (8, 72, 200 columns) they
+    store what they hold.  Large results (the streaming form), sum, mean and max, a column block
+    of a wider matrix: bit-exact against the oracle."""
+    rng = np.random.Generator(np.random.PCG64(dim))
+    rows = 2000
+    n_bags = max(4099, (8 << 20) // (dim * 4) + 3)
+    table = (rng.standard_normal((rows, dim)) * 0.5).astype(np.float16)
+    lengths = rng.integers(0, 4, n_bags)
+    lengths[::1000] = 40
+    idx = rng.integers(0, rows, int(lengths.sum())).astype(np.int32)
+    off = workloads.offsets_from_lengths(lengths, np.int32)
+    assert n_bags * dim * 4 >= 8 << 20
+    for mode in ("sum", "mean", "max"):
+        want, _, _ = oracle.embedding_bag(table, idx, off, OPS[mode], out_dtype=np.float32)
+        got = host(ops.embedding_bag(dev(table), dev(idx), dev(off), mode, out_dtype=torch.float32))
+        assert_bits_equal(got, want, "%s, %d columns" % (mode, dim))
+    wide = torch.full((n_bags, dim + 8), 5.0, dtype=torch.float32, device="cuda")
+    ops.embedding_bag(dev(table), dev(idx), dev(off), "sum", out_dtype=torch.float32, out=wide, out_col=4)
+    w = host(wide)
+    want, _, _ = oracle.embedding_bag(table, idx, off, OPS["sum"], out_dtype=np.float32)
+    assert_bits_equal(w[:, 4:4 + dim], want, "column block")
+    assert (w[:, :4] == 5.0).all() and (w[:, 4 + dim:] == 5.0).all()
+
+
 @pytest.mark.parametrize("tdt,idt", [(np.float16, np.int32), (np.float32, np.int64)])
 def test_ids_and_weights_at_every_alignment(oracle, tdt, idt):
     """A run's ids and weights are staged with 16-byte loads between the first and the last 16-byte

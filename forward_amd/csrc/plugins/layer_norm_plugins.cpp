@@ -98,11 +98,12 @@ LayerNormPluginDynamic* LayerNormPluginDynamic::deserialize(const std::string& n
   ByteReader r(data, length);
   int32_t type = -1, cfg = -1;
   size_t ld = 0;
-  bool has_bias = false;
+  uint8_t bias_byte = 0;  // the reference writes a bool here; read as a byte, since any other value is not a bool to load
   r.pod(&type);
   r.pod(&cfg);
   r.pod(&ld);
-  r.pod(&has_bias);
+  r.pod(&bias_byte);
+  const bool has_bias = bias_byte != 0;
   if (!r.ok()) {
     set_error(FWDMI_ERR_TRUNCATED, "LayerNorm: serialized header truncated");
     return nullptr;

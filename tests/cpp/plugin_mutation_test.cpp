@@ -1,0 +1,254 @@
+// Host-only robustness check of everything that reads engine bytes: every plugin's
+// deserializePlugin and the plan-file loader are fed seeded mutations of valid blobs and files
+// (bytes replaced, bits flipped, pieces cut, repeated or truncated, size fields set to extreme
+// values) and must answer each with NULL and a reason, or with an object that serializes, clones
+// and destroys cleanly.  tests/test_plugin_host.py builds this file and the library's host code with
+// the address / undefined-behaviour sanitizers; no GPU is touched (nothing is configured or enqueued).
+#include <unistd.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "../../include/fwdmi.h"
+
+static int g_failures = 0;
+static long g_alive = 0, g_refused = 0;
+
+#define CHECK(cond, ...)                                               \
+  do {                                                                 \
+    if (!(cond)) {                                                     \
+      std::fprintf(stderr, "FAIL %s:%d: %s: ", __FILE__, __LINE__, #cond); \
+      std::fprintf(stderr, __VA_ARGS__);                               \
+      std::fprintf(stderr, "\n");                                      \
+      ++g_failures;                                                    \
+    }                                                                  \
+  } while (0)
+
+static std::mt19937_64 g_rng(77001);
+static size_t uni(size_t lo, size_t hi) { return std::uniform_int_distribution<size_t>(lo, hi)(g_rng); }
+
+static void mutate(std::vector<char>* t) {
+  static const uint64_t kExtremes[] = {0, 1, 0x7fffffffu, 0x80000000u, 0xffffffffu, 0x100000000ull, 0x7fffffffffffffffull,
+                                       0x8000000000000000ull, 0xffffffffffffffffull, 0xfffffffffffffffeull, 1ull << 40};
+  const int edits = (int)uni(1, 3);
+  for (int e = 0; e < edits && !t->empty(); ++e) {
+    const size_t at = uni(0, t->size() - 1);
+    switch (uni(0, 6)) {
+      case 0: (*t)[at] = (char)uni(0, 255); break;
+      case 1: (*t)[at] ^= (char)(1u << uni(0, 7)); break;
+      case 2: t->erase(t->begin() + (long)at, t->begin() + (long)std::min(t->size(), at + uni(1, 16))); break;
+      case 3: t->resize(at); break;
+      case 4: {  // a piece repeated
+        const size_t n = std::min(t->size() - at, uni(1, 64));
+        const std::vector<char> piece(t->begin() + (long)at, t->begin() + (long)(at + n));
+        t->insert(t->begin() + (long)at, piece.begin(), piece.end());
+        break;
+      }
+      case 5: {  // a 4- or 8-byte field (headers are packed ints and size_t counts) set to an extreme value
+        const size_t w = uni(0, 1) ? 4 : 8, a = std::min(at, t->size() >= w ? t->size() - w : 0) & ~(size_t)3;
+        const uint64_t v = kExtremes[uni(0, sizeof(kExtremes) / sizeof(kExtremes[0]) - 1)];
+        if (a + w <= t->size()) std::memcpy(t->data() + a, &v, w);
+        break;
+      }
+      default: {  // the same, near the start, where the headers are
+        const size_t a = (uni(0, 15) * 4);
+        const uint32_t v = (uint32_t)kExtremes[uni(0, 4)];
+        if (a + 4 <= t->size()) std::memcpy(t->data() + a, &v, 4);
+        break;
+      }
+    }
+  }
+}
+
+// A plugin that came out of damaged bytes must still behave as an object.
+static void exercise(fwdmi_plugin* p) {
+  const size_t n = fwdmi_plugin_get_serialization_size(p);
+  CHECK(n < ((size_t)1 << 28), "serialization size %zu", n);
+  if (n < ((size_t)1 << 28)) {
+    std::vector<char> out(n);  // exact size: a write past it is seen
+    CHECK(fwdmi_plugin_serialize(p, out.data()) == FWDMI_OK, "serialize: %s", fwdmi_last_error());
+  }
+  CHECK(fwdmi_plugin_get_nb_outputs(p) >= 1, "outputs");
+  CHECK(fwdmi_plugin_get_type(p) != nullptr && fwdmi_plugin_get_version(p) != nullptr, "type / version");
+  fwdmi_plugin* c = fwdmi_plugin_clone(p);
+  if (c) {
+    CHECK(fwdmi_plugin_get_serialization_size(c) == n, "a clone serializes to another size");
+    fwdmi_plugin_destroy(c);
+  }
+}
+
+struct Made {
+  const char* name;
+  const char* version;
+  fwdmi_plugin* plugin;
+};
+
+int main() {
+  std::vector<float> gamma(16, 1.0f), beta(16, 0.25f), word(5 * 16, 0.25f), pos(4 * 16, 0.5f), tok(2 * 16, 0.125f);
+  std::vector<float> table(6 * 8, 0.5f), g_rows(8 * 4, 0.5f);
+  const int dim = 8, count = 6, offset = 0, op = 0, ld = 16, f16 = FWDMI_F16, one = 1, g_dim = 4, g_counts[3] = {2, 5, 1};
+  const int i64 = FWDMI_I64;
+  const fwdmi_plugin_field bag[] = {{"dim", &dim, FWDMI_FIELD_I32, 1}, {"count", &count, FWDMI_FIELD_I32, 1},
+                                    {"offset", &offset, FWDMI_FIELD_I32, 1}, {"op", &op, FWDMI_FIELD_I32, 1},
+                                    {"data", table.data(), FWDMI_FIELD_F32, 48}};
+  const fwdmi_plugin_field bag2[] = {bag[0], bag[1], bag[2], bag[3], bag[4], {"index_type", &i64, FWDMI_FIELD_I32, 1},
+                                     {"output_fp16", &one, FWDMI_FIELD_I32, 1}, {"include_last_offset", &one, FWDMI_FIELD_I32, 1},
+                                     {"per_sample_weights", &one, FWDMI_FIELD_I32, 1}};
+  const fwdmi_plugin_field group[] = {{"dim", &g_dim, FWDMI_FIELD_I32, 1}, {"op", &op, FWDMI_FIELD_I32, 1},
+                                      {"count", g_counts, FWDMI_FIELD_I32, 3}, {"data", g_rows.data(), FWDMI_FIELD_F32, 32},
+                                      {"per_sample_weights", &one, FWDMI_FIELD_I32, 1}};
+  const fwdmi_plugin_field ln[] = {{"ld", &ld, FWDMI_FIELD_I32, 1}, {"type_id", &f16, FWDMI_FIELD_I32, 1},
+                                   {"beta", beta.data(), FWDMI_FIELD_F32, 16}, {"gamma", gamma.data(), FWDMI_FIELD_F32, 16},
+                                   {"bias", beta.data(), FWDMI_FIELD_F32, 16}};
+  const float eps = 1e-5f;
+  const fwdmi_plugin_field emb[] = {{"bert_embeddings_layernorm_beta", beta.data(), FWDMI_FIELD_F32, 16},
+                                    {"bert_embeddings_layernorm_gamma", gamma.data(), FWDMI_FIELD_F32, 16},
+                                    {"bert_embeddings_word_embeddings", word.data(), FWDMI_FIELD_F32, 80},
+                                    {"bert_embeddings_token_type_embeddings", tok.data(), FWDMI_FIELD_F32, 32},
+                                    {"bert_embeddings_position_embeddings", pos.data(), FWDMI_FIELD_F32, 64},
+                                    {"output_fp16", &one, FWDMI_FIELD_I32, 1}, {"mha_type_id", &f16, FWDMI_FIELD_I32, 1},
+                                    // the SkipLayerNorm the plugin can also stand for
+                                    {"skip_beta", beta.data(), FWDMI_FIELD_F32, 16}, {"skip_gamma", gamma.data(), FWDMI_FIELD_F32, 16},
+                                    {"skip_bias", beta.data(), FWDMI_FIELD_F32, 16}, {"skip_eps", &eps, FWDMI_FIELD_F32, 1}};
+  struct Recipe {
+    const char* name;
+    const char* version;
+    const fwdmi_plugin_field* fields;
+    int n;
+  } recipes[] = {{"EmbeddingBag_TRT", "001", bag, 5},
+                 {"EmbeddingBag_TRT", "002", bag2, 9},
+                 {"EmbeddingBagGroup_TRT", "001", group, 5},
+                 {"ForwardLayerNormPluginDynamic", "1", ln, 5},
+                 {"CustomSkipLayerNormPluginDynamic", "1", ln, 5},
+                 {"CustomEmbLayerNormPluginDynamic", "1", emb, 7},
+                 {"CustomEmbLayerNormPluginDynamic", "1", emb, 11}};
+
+  std::vector<Made> made;
+  for (const Recipe& r : recipes) {
+    fwdmi_creator* cr = fwdmi_get_plugin_creator(r.name, r.version);
+    CHECK(cr != nullptr, "%s/%s is not registered", r.name, r.version);
+    if (!cr) return 1;
+    fwdmi_plugin* p = fwdmi_creator_create_plugin(cr, "layer", r.fields, r.n);
+    CHECK(p != nullptr, "%s/%s: %s", r.name, r.version, fwdmi_last_error());
+    if (!p) return 1;
+    made.push_back({r.name, r.version, p});
+    std::vector<char> good(fwdmi_plugin_get_serialization_size(p));
+    CHECK(fwdmi_plugin_serialize(p, good.data()) == FWDMI_OK, "serialize");
+    fwdmi_plugin* again = fwdmi_creator_deserialize_plugin(cr, "layer", good.data(), good.size());
+    CHECK(again != nullptr && fwdmi_plugin_get_serialization_size(again) == good.size(), "%s: its own blob", r.name);
+    if (again) fwdmi_plugin_destroy(again);
+    for (size_t n = 0; n < good.size(); ++n) {  // every truncation, from an exact-size heap copy
+      std::vector<char> cut(good.begin(), good.begin() + (long)n);
+      fwdmi_plugin* q = fwdmi_creator_deserialize_plugin(cr, "layer", cut.data(), cut.size());
+      if (q) exercise(q), fwdmi_plugin_destroy(q), ++g_alive;
+      else ++g_refused;
+    }
+    for (int trial = 0; trial < 30000; ++trial) {
+      std::vector<char> bad(good);
+      mutate(&bad);
+      std::vector<char> exact(bad.begin(), bad.end());
+      fwdmi_plugin* q = fwdmi_creator_deserialize_plugin(cr, "layer", exact.data(), exact.size());
+      if (q) {
+        exercise(q);
+        fwdmi_plugin_destroy(q);
+        ++g_alive;
+      } else {
+        CHECK(fwdmi_last_error()[0] != '\0', "%s: refused without a reason", r.name);
+        ++g_refused;
+      }
+    }
+  }
+
+  // ---- plan files -----------------------------------------------------------------------------
+  char dir[] = "/tmp/fwdmi_mutation_XXXXXX";
+  CHECK(mkdtemp(dir) != nullptr, "mkdtemp");
+  const std::string path = std::string(dir) + "/engine.plan", bad_path = std::string(dir) + "/damaged.plan";
+  std::vector<fwdmi_plugin*> handles;
+  std::vector<const char*> names;
+  static const char* const kNames[] = {"bag", "bag2", "group", "ln", "skip_ln", "emb", "emb_skip"};
+  for (size_t i = 0; i < made.size(); ++i) handles.push_back(made[i].plugin), names.push_back(kNames[i]);
+  const char* meta = "{\"infer_mode\":1,\"opt_batch_size\":8,\"max_batch_size\":32,\"torch_module_path\":\"m.pth\","
+                     "\"unused_input_indices\":[1],\"output_indices\":[0,2]}";
+  CHECK(fwdmi_plan_save(path.c_str(), handles.data(), names.data(), (int)handles.size(), meta) == FWDMI_OK, "save: %s",
+        fwdmi_last_error());
+  std::vector<char> file;
+  {
+    FILE* f = std::fopen(path.c_str(), "rb");
+    CHECK(f != nullptr, "open the saved plan");
+    if (f) {
+      char buf[4096];
+      size_t n;
+      while ((n = std::fread(buf, 1, sizeof buf, f)) > 0) file.insert(file.end(), buf, buf + n);
+      std::fclose(f);
+    }
+  }
+  auto load_and_walk = [&](const std::string& where) {
+    fwdmi_plan* plan = fwdmi_plan_load(where.c_str());
+    if (!plan) {
+      CHECK(fwdmi_last_error()[0] != '\0', "plan refused without a reason");
+      ++g_refused;
+      return false;
+    }
+    ++g_alive;
+    const int n = fwdmi_plan_size(plan);
+    CHECK(n >= 0 && n < 100000, "plan of %d entries", n);
+    for (int i = 0; i < n && i < 64; ++i) {
+      CHECK(fwdmi_plan_layer_name(plan, i) != nullptr, "layer name %d", i);
+      fwdmi_plugin* p = fwdmi_plan_take_plugin(plan, i);
+      if (p) exercise(p), fwdmi_plugin_destroy(p);
+      CHECK(fwdmi_plan_take_plugin(plan, i) == nullptr, "entry %d handed out twice", i);
+    }
+    CHECK(fwdmi_plan_meta(plan) != nullptr, "meta text");
+    fwdmi_meta* m = fwdmi_plan_meta_data(plan);
+    if (m) fwdmi_meta_free(m);
+    fwdmi_plan_close(plan);
+    return true;
+  };
+  CHECK(load_and_walk(path), "the saved plan does not load: %s", fwdmi_last_error());
+  // the sidecar of the damaged copies: sometimes the good one, sometimes damaged, sometimes none
+  std::vector<char> meta_file;
+  {
+    FILE* f = std::fopen((path + ".meta").c_str(), "rb");
+    CHECK(f != nullptr, "the sidecar was not written");
+    if (f) {
+      char buf[4096];
+      size_t n;
+      while ((n = std::fread(buf, 1, sizeof buf, f)) > 0) meta_file.insert(meta_file.end(), buf, buf + n);
+      std::fclose(f);
+    }
+  }
+  auto write_file = [](const std::string& where, const std::vector<char>& bytes) {
+    FILE* f = std::fopen(where.c_str(), "wb");
+    if (!f) return false;
+    const bool ok = bytes.empty() || std::fwrite(bytes.data(), 1, bytes.size(), f) == bytes.size();
+    return std::fclose(f) == 0 && ok;
+  };
+  for (int trial = 0; trial < 6000; ++trial) {
+    std::vector<char> bad(file);
+    if (trial % 3 != 2) mutate(&bad);
+    CHECK(write_file(bad_path, bad), "write the damaged plan");
+    const int kind = trial % 3;
+    if (kind == 0) {
+      CHECK(write_file(bad_path + ".meta", meta_file), "write the sidecar");
+    } else if (kind == 1) {
+      std::remove((bad_path + ".meta").c_str());
+    } else {
+      std::vector<char> bad_meta(meta_file);
+      mutate(&bad_meta);
+      CHECK(write_file(bad_path + ".meta", bad_meta), "write the damaged sidecar");
+    }
+    load_and_walk(bad_path);
+  }
+  std::remove(bad_path.c_str());
+  std::remove((bad_path + ".meta").c_str());
+  std::remove(path.c_str());
+  std::remove((path + ".meta").c_str());
+  rmdir(dir);
+  for (const Made& m : made) fwdmi_plugin_destroy(m.plugin);
+  std::printf("%ld damaged inputs gave an object, %ld were refused, %d failures\n", g_alive, g_refused, g_failures);
+  return g_failures ? 1 : 0;
+}

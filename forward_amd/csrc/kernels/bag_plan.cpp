@@ -43,8 +43,9 @@ int bag_plan(const fwdmi_bag_table* tables_dev, const fwdmi_bag_table* tables_in
   if (op != FWDMI_OP_SUM && op != FWDMI_OP_MEAN && op != FWDMI_OP_MAX && op != FWDMI_OP_SQUARE_SUM)
     return set_error(FWDMI_ERR_UNSUPPORTED, "embedding bag: unknown op %d", op);
   // dim: a row's byte size and a run's (bag, slice) count stay far inside 32 bits
-  FWDMI_REQUIRE(n_bags >= 0 && dim > 0 && dim <= (1 << 24) && n_tables > 0,
-                "embedding bag: n_bags=%lld dim=%d (1 .. 2^24) n_tables=%d", (long long)n_bags, dim, n_tables);
+  // n_tables: the per-table passes below stay short whatever a caller passes
+  FWDMI_REQUIRE(n_bags >= 0 && dim > 0 && dim <= (1 << 24) && n_tables > 0 && n_tables <= (1 << 20),
+                "embedding bag: n_bags=%lld dim=%d (1 .. 2^24) n_tables=%d (1 .. 2^20)", (long long)n_bags, dim, n_tables);
   FWDMI_REQUIRE(!(x.per_sample_weights || (multi && (x.flags & FWDMI_BAG_TABLE_WEIGHTS))) || op == FWDMI_OP_SUM,
                 "embedding bag: per_sample_weights needs op SUM (got %d)", op);
   FWDMI_REQUIRE(!x.max_indices || (op == FWDMI_OP_MAX && !multi),
@@ -60,7 +61,7 @@ int bag_plan(const fwdmi_bag_table* tables_dev, const fwdmi_bag_table* tables_in
     FWDMI_REQUIRE(single.input_size >= 0 && (single.input_size == 0 || single.input),
                   "embedding bag: null ids");
     FWDMI_REQUIRE(fixed_len >= 0 || single.input_2, "embedding bag: null offsets");
-    FWDMI_REQUIRE(single.out_col >= 0 && single.out_col + dim <= out_stride, "embedding bag: out_col");
+    FWDMI_REQUIRE(single.out_col >= 0 && single.out_col <= out_stride - dim, "embedding bag: out_col");
   }
 
   const size_t sw = dtype_size(x.table_dtype), so = dtype_size(x.out_dtype);
@@ -171,8 +172,9 @@ int bag_plan(const fwdmi_bag_table* tables_dev, const fwdmi_bag_table* tables_in
       L.idx_cap = cap_max;
     }
   }
-  const int64_t wgs = (n_bags + L.bags_per_wg - 1) / L.bags_per_wg;
-  FWDMI_REQUIRE(wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
+  auto runs_of = [&](int per_run) { return n_bags / per_run + (n_bags % per_run != 0); };  // no sum that could overflow
+  const int64_t wgs = runs_of(L.bags_per_wg);
+  FWDMI_REQUIRE(wgs < (int64_t)1 << 31 && wgs * n_tables < (int64_t)1 << 31, "embedding bag: grid too large");
   L.wgs_per_table = (int)wgs;
   int64_t total_runs = wgs * n_tables;
   L.var_runs = 0;
@@ -181,7 +183,9 @@ int bag_plan(const fwdmi_bag_table* tables_dev, const fwdmi_bag_table* tables_in
     for (int t = 0; t < n_tables; ++t) {
       L.run_start[t] = (int32_t)total_runs;
       L.run_bags[t] = (uint16_t)run_bags[t];
-      total_runs += (n_bags + run_bags[t] - 1) / run_bags[t];
+      const int64_t runs_t = runs_of(run_bags[t]);
+      FWDMI_REQUIRE(runs_t < (int64_t)1 << 31, "embedding bag: grid too large");
+      total_runs += runs_t;
       FWDMI_REQUIRE(total_runs < (int64_t)1 << 31, "embedding bag: grid too large");
     }
     L.run_start[n_tables] = (int32_t)total_runs;

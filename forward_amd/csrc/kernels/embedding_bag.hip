@@ -886,14 +886,17 @@ int check_host_tables(const char* what, const fwdmi_bag_table* tables_host, int3
   const size_t sw = ext ? fwdmi::dtype_size(ext->table_dtype) : sizeof(float);
   const size_t so = ext ? fwdmi::dtype_size(ext->out_dtype) : sizeof(float);
   const int64_t stride = ext && ext->out_row_stride > 0 ? ext->out_row_stride : dim;
+  if (ext && (!fwdmi::is_float_dtype(ext->table_dtype) || !fwdmi::is_float_dtype(ext->out_dtype)))  // sizes of 0 below otherwise
+    return fwdmi::set_error(FWDMI_ERR_UNSUPPORTED, "%s: unsupported dtype (table %d, out %d)", what, ext->table_dtype,
+                            ext->out_dtype);
   for (int32_t t = 0; t < n_tables; ++t) {
     const fwdmi_bag_table& d = tables_host[t];
     FWDMI_REQUIRE(d.count <= 0 || d.data, "%s: table %d has rows but no data", what, t);
     FWDMI_REQUIRE(d.input_size >= 0 && (d.input_size == 0 || d.input) && d.input_2, "%s: table %d lacks ids or offsets", what, t);
-    FWDMI_REQUIRE(d.out_col >= 0 && dim > 0 && d.out_col + dim <= stride,
+    FWDMI_REQUIRE(d.out_col >= 0 && dim > 0 && stride >= dim && d.out_col <= stride - dim,
                   "%s: table %d writes columns %lld.. beyond the row of %lld", what, t, (long long)d.out_col,
                   (long long)stride);
-    if (sw && ((size_t)dim * sw) % 16 == 0) {  // rows are read (and written) as 16-byte slices
+    if (((size_t)dim * sw) % 16 == 0) {  // rows are read (and written) as 16-byte slices
       const size_t store_align = std::min<size_t>(16, 16 / sw * so);
       FWDMI_REQUIRE(reinterpret_cast<uintptr_t>(d.data) % 16 == 0 && ((size_t)d.out_col * so) % store_align == 0,
                     "%s: table %d: data or output column not aligned to its slices", what, t);

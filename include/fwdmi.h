@@ -175,7 +175,7 @@ typedef struct fwdmi_bag_table {
  * one [n_bags, out_row_stride] matrix.  Equivalent to n_tables calls of fwdmi_embedding_bag
  * with ext->out_row_stride set (the reference issues one plugin enqueue per table,
  * embedding_bag_plugin.cpp:146-189, and concatenates afterwards).
- * `avg_bag_len` (>0) is a sizing hint: the mean ids per bag over the batch.
+ * `avg_bag_len` (>0) is a sizing hint: the mean ids per bag over the batch.  At most 2^20 tables per launch.
  * Per-sample weights come through the descriptors (FWDMI_BAG_TABLE_WEIGHTS), not through
  * ext->per_sample_weights; max_indices is not available in this form.
  */

@@ -3,7 +3,9 @@
 // that every bag of every table is reduced exactly once, that nothing reaches past the tables'
 // bags or the LDS carve-up, and that the per-die segments are what the plan says.
 // Built with g++ and the address / undefined-behaviour sanitizers by tests/test_bag_plan.py.
+#include <climits>
 #include <cmath>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -315,6 +317,74 @@ int main() {
     c.n_tables = kInlineTables + 1;
     c.name = "too many inline tables";
     expect_error(c, "do not fit");
+  }
+  // Arguments at the ends of their types, in every combination the generator hits: the plan either
+  // refuses them with a reason or is a plan; the sanitizers this file is built with see any signed
+  // overflow, out-of-range conversion or read past an array on the way.
+  {
+    static const int dummy[64] = {};
+    alignas(16) static char out[16];
+    const int64_t bags[] = {-1, 0, 1, 7, 65536, 2147483647, 2147483648ll, (int64_t)1 << 40, (int64_t)1 << 62, INT64_MAX};
+    const int64_t lens[] = {-1, -1, -1, 0, 1, 40, 2147483648ll, (int64_t)1 << 62, INT64_MAX};
+    const int dims[] = {-1, 0, 1, 8, 128, 1 << 20, 1 << 30, INT32_MAX};
+    const int tables[] = {-1, 0, 1, 2, 26, 64, 65, 1024, 2048, 100000, INT32_MAX};
+    const double avgs[] = {std::nan(""), INFINITY, -INFINITY, 0.0, 1.0, 16.0, 1e308, -1e308, 5e-324};
+    const int ops[] = {-1, 0, 1, 2, 3, 4, 999, 12345, INT32_MAX};
+    const int types[] = {FWDMI_F32, FWDMI_F16, FWDMI_I8, FWDMI_I32, FWDMI_I64, -1, 77};
+    const int64_t strides[] = {0, 0, 1, 128, 3328, -5, (int64_t)1 << 40, INT64_MAX};
+    const int cus[] = {-1, 0, 1, 32, 256, 304, 1 << 30, INT32_MAX}, xcds[] = {-1, 0, 1, 2, 8, 9, 1 << 30};
+    long refused = 0, planned = 0;
+    std::vector<float> ones(2048, 1.0f), wild(2048);
+    for (size_t i = 0; i < wild.size(); ++i) wild[i] = (i % 5 == 0) ? 3e38f : (float)(i % 300);
+#define ANY(a) a[rng() % (sizeof(a) / sizeof(a[0]))]
+    // mostly plausible values, so that the extreme ones get past the first checks one or two at a time
+    const int64_t sane_bags[] = {1, 7, 1000, 65536, 3000000}, sane_lens[] = {-1, -1, -1, 0, 1, 40}, sane_strides[] = {0, 0, 0, 1 << 20};
+    const int sane_dims[] = {1, 8, 64, 128, 1000, 4096}, sane_tables[] = {1, 2, 26, 40, 41, 64, 65, 700};
+    const double sane_avgs[] = {0.5, 1.0, 16.3, 300.0};
+    const int sane_ops[] = {0, 0, 1, 2, 3}, sane_types[] = {FWDMI_F32, FWDMI_F16}, sane_cus[] = {256, 256, 32, 304}, sane_xcds[] = {8, 8, 1, 4};
+#define PICK(a) (uni(0, 5) ? ANY(sane_##a) : ANY(a))
+    for (int it = 0; it < 200000; ++it) {
+      const int n_tables = PICK(tables), form = uni(0, 2);
+      fwdmi_bag_ext x{};
+      x.table_dtype = PICK(types);
+      x.index_dtype = uni(0, 3) ? (uni(0, 1) ? FWDMI_I32 : FWDMI_I64) : PICK(types);
+      x.out_dtype = uni(0, 3) ? (uni(0, 1) ? FWDMI_F32 : FWDMI_F16) : PICK(types);
+      x.include_last_offset = uni(0, 2) - 1;
+      x.out_row_stride = PICK(strides);
+      x.flags = uni(0, 7);
+      const bool arrays_fit = n_tables > 0 && n_tables <= 2048;
+      if (arrays_fit && uni(0, 1)) x.table_cost = uni(0, 1) ? ones.data() : wild.data();
+      if (arrays_fit && (x.flags & FWDMI_BAG_TABLE_AVG_LEN) && uni(0, 1)) x.table_avg_len = uni(0, 1) ? ones.data() : wild.data();
+      if (!arrays_fit) x.flags &= ~FWDMI_BAG_TABLE_AVG_LEN, x.table_avg_len = nullptr;
+      if (uni(0, 5) == 0) x.per_sample_weights = dummy;
+      if (uni(0, 5) == 0) x.max_indices = out;
+      if (uni(0, 5) == 0) x.square_sum_out = out;
+      fwdmi_bag_table single{uni(0, 9) ? dummy : nullptr, uni(0, 9) ? dummy : nullptr, uni(0, 9) ? dummy : nullptr,
+                             PICK(bags), PICK(bags), PICK(lens), PICK(strides), nullptr};
+      std::vector<fwdmi_bag_table> inl;
+      if (form == 2 && n_tables > 0 && n_tables <= kInlineTables) inl.assign((size_t)n_tables, single);
+      const fwdmi_bag_table* dev = form == 1 ? reinterpret_cast<const fwdmi_bag_table*>(dummy) : nullptr;
+      const BagTopology tp{PICK(cus), PICK(xcds)};
+      BagPlan P;
+      const int rc = bag_plan(dev, inl.empty() ? nullptr : inl.data(), form == 0 ? 1 : n_tables, single, uni(0, 9) ? out : nullptr,
+                              PICK(bags), PICK(lens), PICK(dims), PICK(ops), PICK(avgs), uni(0, 9) ? &x : nullptr, tp, &P);
+      if (rc != FWDMI_OK) {
+        ++refused;
+        if (fwdmi_last_error()[0] == '\0') {
+          std::fprintf(stderr, "FAIL extreme arguments #%d: refused without a reason\n", it);
+          ++g_failures;
+        }
+      } else {
+        ++planned;
+        if (!P.empty && (P.grid <= 0 || P.block <= 0 || P.lds > (size_t)kBagLdsLimit)) {
+          std::fprintf(stderr, "FAIL extreme arguments #%d: grid %d block %d lds %zu\n", it, P.grid, P.block, P.lds);
+          ++g_failures;
+        }
+      }
+    }
+#undef PICK
+#undef ANY
+    std::printf("extreme arguments: %ld refused, %ld planned\n", refused, planned);
   }
   std::printf("%ld plans walked, %d failures\n", g_plans, g_failures);
   return g_failures ? 1 : 0;

@@ -2,10 +2,13 @@
 // deserializePlugin and the plan-file loader are fed seeded mutations of valid blobs and files
 // (bytes replaced, bits flipped, pieces cut, repeated or truncated, size fields set to extreme
 // values) and must answer each with NULL and a reason, or with an object that serializes, clones
-// and destroys cleanly.  tests/test_plugin_host.py builds this file and the library's host code with
+// and destroys cleanly.  Then the kernel launchers are called with arguments at the ends of their
+// types: without a device each call must return a status.  tests/test_plugin_host.py builds this file and the library's host code with
 // the address / undefined-behaviour sanitizers; no GPU is touched (nothing is configured or enqueued).
 #include <unistd.h>
 
+#include <climits>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -249,6 +252,95 @@ int main() {
   std::remove((path + ".meta").c_str());
   rmdir(dir);
   for (const Made& m : made) fwdmi_plugin_destroy(m.plugin);
-  std::printf("%ld damaged inputs gave an object, %ld were refused, %d failures\n", g_alive, g_refused, g_failures);
+
+  // ---- launchers with arguments at the ends of their types ---------------------------------------
+  // Without a device every launcher must come back with a status: its argument checks and sizing
+  // arithmetic run on the host before anything is enqueued, and the sanitizers see them.  (With a
+  // device present this part is skipped: the pointers below are not device memory.)
+  long statuses = 0, nothing_to_do = 0;
+  if (fwdmi_device_count() == 0) {
+    alignas(16) static char mem[256];
+    const int64_t big[] = {-1, 0, 1, 7, 768, 1024, 65536, 2147483647, 2147483648ll, (int64_t)1 << 40, (int64_t)1 << 62, INT64_MAX};
+    const int32_t small[] = {-1, 0, 1, 2, 8, 128, 768, 1024, 16384, 1 << 24, 1 << 30, INT32_MAX};
+    const int32_t types[] = {FWDMI_F32, FWDMI_F16, FWDMI_F32, FWDMI_F16, FWDMI_I8, FWDMI_I32, FWDMI_I64, -1, 99};
+    const int32_t ops[] = {0, 1, 2, 3, 0, 999, -1, 12345};
+    const float epss[] = {0.0f, 1e-12f, 1e-5f, -1.0f, 3e38f, -3e38f};
+#define PICK(a) a[uni(0, sizeof(a) / sizeof(a[0]) - 1)]
+    auto ptr = [&]() -> void* { return uni(0, 7) ? (void*)mem : nullptr; };
+    for (int it = 0; it < 100000; ++it) {
+      int rc = 1;
+      fwdmi_bag_ext x{};
+      x.table_dtype = PICK(types), x.index_dtype = uni(0, 2) ? (uni(0, 1) ? FWDMI_I32 : FWDMI_I64) : PICK(types);
+      x.out_dtype = PICK(types), x.include_last_offset = (int32_t)uni(0, 1), x.out_row_stride = uni(0, 2) ? 0 : PICK(big);
+      x.flags = (int32_t)uni(0, 7) & ~FWDMI_BAG_TABLE_AVG_LEN;
+      x.per_sample_weights = uni(0, 5) ? nullptr : mem, x.max_indices = uni(0, 5) ? nullptr : mem;
+      x.square_sum_out = uni(0, 5) ? nullptr : mem, x.oob_flag = uni(0, 3) ? nullptr : (int32_t*)mem;
+      const fwdmi_bag_ext* xp = uni(0, 4) ? &x : nullptr;
+      bool empty_work = false;  // FWDMI_OK is the answer to a call that has nothing to do: no launch, no device needed
+      const int64_t n0 = PICK(big), n1 = PICK(big), n2 = PICK(big), n3 = PICK(big);
+      const int32_t s0 = PICK(small), s1 = PICK(small), s2 = PICK(small);
+      switch (uni(0, 8)) {
+        case 0: rc = fwdmi_layer_norm(nullptr, s0, n0, ptr(), (float*)ptr(), (float*)ptr(), ptr(), (float*)ptr(),
+                                      PICK(types), PICK(epss));
+                empty_work = n0 == 0;
+                break;
+        case 1: rc = fwdmi_skip_layer_norm(nullptr, s0, n0, ptr(), ptr(), (float*)ptr(), (float*)ptr(), ptr(),
+                                           (float*)ptr(), PICK(types), PICK(epss));
+                empty_work = n0 == 0;
+                break;
+        case 2: {
+          fwdmi_emb_ext e{(int32_t)uni(0, 1), PICK(epss), ptr(), (float*)ptr(), (float*)ptr(), (float*)ptr(), ptr()};
+          rc = fwdmi_emb_layer_norm_ex(nullptr, s0, s1, s2, (int32_t*)ptr(), (int32_t*)ptr(),
+                                       (int32_t*)ptr(), (float*)ptr(), (float*)ptr(), ptr(), ptr(), ptr(), PICK(small), PICK(small),
+                                       PICK(small), ptr(), (int32_t*)ptr(), PICK(types), PICK(epss), (int32_t*)ptr(),
+                                       uni(0, 1) ? &e : nullptr);
+          empty_work = s0 == 0 || s1 == 0;
+          break;
+        }
+        case 3: rc = fwdmi_embedding_bag(ptr(), ptr(), ptr(), n0, n1, ptr(), n2, s0, n3, PICK(ops), xp, nullptr);
+                empty_work = n1 == 0;
+                break;
+        case 4: rc = fwdmi_embedding_bag_fixed(ptr(), ptr(), n0, n1, ptr(), n2, s0, n3, PICK(ops), xp, nullptr);
+                empty_work = n0 == 0;
+                break;
+        case 5: rc = fwdmi_gather(ptr(), ptr(), n0, n1, ptr(), n2, s0, n3, xp, nullptr);
+                empty_work = n0 == 0 || n1 == 0;
+                break;
+        case 6:
+        case 7: {
+          const int n = (int)uni(0, 70);
+          std::vector<fwdmi_bag_table> t((size_t)n);
+          for (auto& d : t) d = fwdmi_bag_table{ptr(), ptr(), ptr(), PICK(big), PICK(big), PICK(big), PICK(big), ptr()};
+          const int32_t n_arg = uni(0, 9) ? n : PICK(small);
+          if (n_arg > n || n_arg < 0) {  // a count beyond the array: only the forms that refuse it before reading
+            rc = fwdmi_embedding_bag_multi_host(nullptr, n_arg, nullptr, n0, ptr(), s0, PICK(ops), 4.0, xp, nullptr);
+          } else if (uni(0, 1)) {
+            rc = fwdmi_embedding_bag_multi_host(t.data(), n_arg, (fwdmi_bag_table*)ptr(), n0, ptr(), s0, PICK(ops),
+                                                uni(0, 3) ? 4.0 : (double)PICK(big), xp, nullptr);
+          } else {
+            rc = fwdmi_embedding_bag_multi_noalloc(t.data(), n_arg, n0, ptr(), s0, PICK(ops), 4.0, xp, nullptr);
+          }
+          empty_work = n0 == 0;
+          break;
+        }
+        default: {
+          const int n = (int)uni(0, 70);
+          std::vector<int64_t> bytes((size_t)n);
+          for (auto& b : bytes) b = PICK(big);
+          std::vector<float> cost((size_t)n + 1);
+          rc = fwdmi_bag_table_cost(uni(0, 9) ? bytes.data() : nullptr, uni(0, 9) ? n : -n, uni(0, 9) ? cost.data() : nullptr);
+          if (rc == FWDMI_OK) rc = -100;  // the one call here that can succeed without a device
+          break;
+        }
+      }
+      CHECK(rc < 0 || (rc == FWDMI_OK && empty_work), "launcher call #%d returned %d without a device", it, rc);
+      CHECK(rc == -100 || rc == FWDMI_OK || fwdmi_last_error()[0] != '\0', "launcher call #%d: status %d without a reason", it, rc);
+      if (rc == FWDMI_OK) ++nothing_to_do;
+      ++statuses;
+    }
+#undef PICK
+  }
+  std::printf("%ld damaged inputs gave an object, %ld were refused, %ld launcher calls without a device returned a status (%ld had nothing to do), %d failures\n",
+              g_alive, g_refused, statuses, nothing_to_do, g_failures);
   return g_failures ? 1 : 0;
 }

@@ -70,9 +70,14 @@ Dims EmbeddingBagPlugin::getOutputDimensions(int outputIndex, const Dims* inputs
     set_error(FWDMI_ERR_UNSUPPORTED, "EmbeddingBag: GATHER with an offsets input is not supported");
     return error_dims();
   }
+  const int n_off = off.nbDims == 1 ? off.d[0] : off.d[1], trailing = opt_.include_last_offset ? 1 : 0;
+  if (n_off < trailing) {
+    set_error(FWDMI_ERR_BAD_ARG, "EmbeddingBag: %d offsets", n_off);
+    return error_dims();
+  }
   Dims out{};
   out.nbDims = 2;
-  out.d[0] = (off.nbDims == 1 ? off.d[0] : off.d[1]) - (opt_.include_last_offset ? 1 : 0);
+  out.d[0] = n_off - trailing;
   out.d[1] = dim_;
   return out;
 }

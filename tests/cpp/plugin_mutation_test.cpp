@@ -166,6 +166,115 @@ int main() {
     }
   }
 
+  // ---- shape, format and type queries with arguments no builder would send -----------------------
+  // Everything here is host code of a plugin that was never configured: it must answer (or refuse)
+  // without reading past its arguments or overflowing on the way.
+  {
+    const int32_t ds[] = {-1, 0, 1, 2, 5, 16, 128, 65536, 1 << 30, INT32_MAX, INT32_MIN};
+    const int32_t ts[] = {FWDMI_F32, FWDMI_F16, FWDMI_I8, FWDMI_I32, FWDMI_BOOL, FWDMI_I64, -1, 1000};
+    auto pick_d = [&]() { return ds[uni(0, sizeof(ds) / sizeof(ds[0]) - 1)]; };
+    auto pick_t = [&]() { return ts[uni(0, sizeof(ts) / sizeof(ts[0]) - 1)]; };
+    long answered = 0;
+    for (const Made& m : made) {
+      for (int it = 0; it < 20000; ++it) {
+        fwdmi_dims in[8];
+        fwdmi_tensor_desc io[12];
+        for (auto& d : in) {
+          d.nbDims = uni(0, 9) ? (int32_t)uni(0, 8) : pick_d();
+          for (auto& v : d.d) v = uni(0, 2) ? (int32_t)uni(1, 64) : pick_d();
+        }
+        for (auto& t : io) {
+          t.dims = in[uni(0, 7)];
+          t.type = pick_t();
+          t.format = uni(0, 5) ? FWDMI_FORMAT_LINEAR : pick_d();
+          t.scale = 1.0f;
+        }
+        const int nb_in = uni(0, 9) ? (int)uni(0, 6) : pick_d(), nb_out = uni(0, 9) ? (int)uni(0, 3) : pick_d();
+        fwdmi_dims out{};
+        // counts beyond the arrays above are only sent where the callee looks at the count first
+        const int in_ok = nb_in >= 0 && nb_in <= 8 ? nb_in : 0, out_ok = nb_out >= 0 && nb_out <= 4 ? nb_out : 0;
+        (void)fwdmi_plugin_get_output_dimensions(m.plugin, uni(0, 5) ? (int)uni(0, 2) : pick_d(), in, in_ok, &out);
+        (void)fwdmi_plugin_get_output_dimensions(m.plugin, 0, uni(0, 9) ? in : nullptr, in_ok, uni(0, 9) ? &out : nullptr);
+        (void)fwdmi_plugin_supports_format_combination(m.plugin, uni(0, 5) ? (int)uni(0, 6) : pick_d(), io, in_ok, out_ok);
+        (void)fwdmi_plugin_get_workspace_size(m.plugin, io, in_ok, io + in_ok, out_ok);
+        int32_t types[8];
+        for (auto& t : types) t = pick_t();
+        (void)fwdmi_plugin_get_output_data_type(m.plugin, uni(0, 5) ? (int)uni(0, 2) : pick_d(), types, in_ok);
+        const void* ins[8] = {};
+        void* outs[4] = {};
+        const int rc = fwdmi_plugin_enqueue(m.plugin, io, io + in_ok, ins, outs, nullptr, nullptr);
+        CHECK(rc < 0, "%s: enqueue on a plugin that was never configured returned %d", m.name, rc);
+        ++answered;
+      }
+    }
+    std::printf("%ld rounds of shape / format / type queries answered\n", answered);
+  }
+
+  // ---- null handles: a status, NULL or an empty answer, never a dereference -------------------------
+  {
+    fwdmi_dims d{};
+    fwdmi_tensor_desc t{};
+    int32_t ty = 0;
+    const int32_t* arr = nullptr;
+    CHECK(fwdmi_get_plugin_creator(nullptr, nullptr) == nullptr, "creator of no name");
+    CHECK(fwdmi_get_plugin_creator("EmbeddingBag_TRT", nullptr) == nullptr, "creator of no version");
+    CHECK(fwdmi_registry_at(-1) == nullptr && fwdmi_registry_at(fwdmi_registry_size()) == nullptr, "registry index");
+    (void)fwdmi_creator_name(nullptr), (void)fwdmi_creator_version(nullptr), (void)fwdmi_creator_num_fields(nullptr);
+    (void)fwdmi_creator_field_name(nullptr, 0), (void)fwdmi_creator_field_type(nullptr, 0);
+    fwdmi_creator* cr = fwdmi_get_plugin_creator("EmbeddingBag_TRT", "001");
+    (void)fwdmi_creator_field_name(cr, -1), (void)fwdmi_creator_field_name(cr, 1000), (void)fwdmi_creator_field_type(cr, -1);
+    CHECK(fwdmi_creator_create_plugin(nullptr, "x", nullptr, 0) == nullptr, "plugin of no creator");
+    CHECK(fwdmi_creator_create_plugin(cr, nullptr, nullptr, 5) == nullptr, "plugin of no fields");
+    CHECK(fwdmi_creator_deserialize_plugin(nullptr, "x", "abc", 3) == nullptr, "blob for no creator");
+    CHECK(fwdmi_creator_deserialize_plugin(cr, "x", nullptr, 100) == nullptr, "no blob");
+    CHECK(fwdmi_plugin_get_nb_outputs(nullptr) < 0, "outputs of no plugin");
+    CHECK(fwdmi_plugin_get_output_dimensions(nullptr, 0, &d, 1, &d) < 0, "dims of no plugin");
+    CHECK(fwdmi_plugin_supports_format_combination(nullptr, 0, &t, 1, 1) <= 0, "formats of no plugin");
+    CHECK(fwdmi_plugin_configure(nullptr, &t, 1, &t, 1) < 0, "configure no plugin");
+    (void)fwdmi_plugin_get_workspace_size(nullptr, &t, 1, &t, 1);
+    CHECK(fwdmi_plugin_initialize(nullptr) < 0, "initialize no plugin");
+    fwdmi_plugin_terminate(nullptr);
+    CHECK(fwdmi_plugin_enqueue(nullptr, &t, &t, nullptr, nullptr, nullptr, nullptr) < 0, "enqueue no plugin");
+    (void)fwdmi_plugin_get_serialization_size(nullptr);
+    CHECK(fwdmi_plugin_serialize(nullptr, &d) < 0, "serialize no plugin");
+    CHECK(fwdmi_plugin_serialize(made[0].plugin, nullptr) < 0, "serialize into nothing");
+    (void)fwdmi_plugin_get_type(nullptr), (void)fwdmi_plugin_get_version(nullptr), (void)fwdmi_plugin_get_namespace(nullptr);
+    fwdmi_plugin_set_namespace(nullptr, "x");
+    fwdmi_plugin_set_namespace(made[0].plugin, nullptr);
+    CHECK(fwdmi_plugin_get_output_data_type(nullptr, 0, &ty, 1) < 0, "type of no plugin");
+    CHECK(fwdmi_plugin_clone(nullptr) == nullptr, "clone of no plugin");
+    fwdmi_plugin_destroy(nullptr);
+    CHECK(fwdmi_plugin_take_oob_flag(nullptr, nullptr) < 0, "flag of no plugin");
+    CHECK(fwdmi_plan_save(nullptr, nullptr, nullptr, 0, nullptr) < 0, "plan without a path");
+    CHECK(fwdmi_plan_save("/tmp/fwdmi_never_written.plan", nullptr, nullptr, 3, nullptr) < 0, "plan of no plugins");
+    CHECK(fwdmi_plan_load(nullptr) == nullptr, "plan of no path");
+    CHECK(fwdmi_plan_size(nullptr) <= 0, "size of no plan");
+    (void)fwdmi_plan_layer_name(nullptr, 0);
+    CHECK(fwdmi_plan_take_plugin(nullptr, 0) == nullptr, "plugin of no plan");
+    (void)fwdmi_plan_meta(nullptr);
+    CHECK(fwdmi_plan_meta_data(nullptr) == nullptr, "sidecar of no plan");
+    fwdmi_plan_close(nullptr);
+    CHECK(fwdmi_meta_load(nullptr) == nullptr && fwdmi_meta_parse(nullptr) == nullptr, "sidecar of nothing");
+    CHECK(fwdmi_meta_save(nullptr, "/tmp/x") < 0, "save no sidecar");
+    (void)fwdmi_meta_json(nullptr), (void)fwdmi_meta_infer_mode(nullptr), (void)fwdmi_meta_opt_batch_size(nullptr);
+    (void)fwdmi_meta_max_batch_size(nullptr), (void)fwdmi_meta_torch_module_path(nullptr);
+    (void)fwdmi_meta_unused_input_indices(nullptr, &arr), (void)fwdmi_meta_output_indices(nullptr, nullptr);
+    CHECK(fwdmi_meta_set(nullptr, 0, 1, 1, nullptr, 0, nullptr, 0, nullptr) < 0, "set no sidecar");
+    fwdmi_meta* m = fwdmi_meta_new();
+    CHECK(m != nullptr, "a new sidecar");
+    if (m) {
+      CHECK(fwdmi_meta_set(m, 0, 1, 1, nullptr, 3, nullptr, 0, nullptr) < 0, "three indices from no array");
+      CHECK(fwdmi_meta_set(m, 0, 1, 1, nullptr, -1, nullptr, -1, nullptr) < 0, "negative counts");
+      CHECK(fwdmi_meta_save(m, nullptr) < 0, "save to no path");
+      fwdmi_meta_free(m);
+    }
+    fwdmi_meta_free(nullptr);
+    int32_t cus = 0;
+    (void)fwdmi_bag_device_topology(nullptr, nullptr), (void)fwdmi_bag_device_topology(&cus, nullptr);
+    CHECK(fwdmi_bag_tables_fill(nullptr, 3, nullptr, nullptr) < 0, "fill from nothing");
+    CHECK(fwdmi_bag_table_cost(nullptr, 3, nullptr) < 0, "cost of nothing");
+  }
+
   // ---- plan files -----------------------------------------------------------------------------
   char dir[] = "/tmp/fwdmi_mutation_XXXXXX";
   CHECK(mkdtemp(dir) != nullptr, "mkdtemp");

@@ -163,11 +163,22 @@ __device__ __forceinline__ void mask_index_wave(const LnLaunch& L, int b, int la
   int first = L.S;
   const int64_t base = L.batch_major ? (int64_t)b * L.S : b;
   const int64_t step = L.batch_major ? 1 : L.B;
-  for (int s = lane; s < L.S; s += 64)
-    if (L.input_mask[base + (int64_t)s * step] == 0) {
-      first = s;
-      break;
+  // Eight positions per lane are read before the first is looked at: one trip to memory for
+  // sequences of up to 512 positions instead of one per 64 (the kernel lasts as long as its slowest
+  // wavefront, and in sequence-major layout every one of these loads is a cache line of its own).
+  constexpr int kAhead = 8;
+  for (int s0 = lane; s0 < L.S; s0 += 64 * kAhead) {
+    int v[kAhead];
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+      const int s = s0 + 64 * k;
+      v[k] = s < L.S ? L.input_mask[base + (int64_t)s * step] : 1;
     }
+#pragma unroll
+    for (int k = kAhead - 1; k >= 0; --k)
+      if (v[k] == 0) first = s0 + 64 * k;  // descending: the earliest position is assigned last
+    if (__builtin_amdgcn_ballot_w64(first != L.S) != 0) break;  // a zero in this block: none earlier remains unseen
+  }
   first = wave_min(first);
   if (lane == 0) L.mask_idx[b] = first;
 }

@@ -36,6 +36,17 @@ __device__ __forceinline__ Pack<T, N> gload(const T FWDMI_GLOBAL* p) {
   }
   return r;
 }
+// The same load with the non-temporal hint, for data that is read once (a run's ids and weights):
+// the lines pass through L2 without taking the place of table rows.
+template <typename T, int N>
+__device__ __forceinline__ Pack<T, N> gload_stream(const T FWDMI_GLOBAL* p) {
+  static_assert(N > 1, "vector loads only");
+  typedef T V __attribute__((ext_vector_type(N), aligned(alignof(Pack<T, N>))));
+  const V x = __builtin_nontemporal_load((const V FWDMI_GLOBAL*)p);
+  Pack<T, N> r;
+  __builtin_memcpy(&r, &x, sizeof(r));
+  return r;
+}
 template <typename T, int N>
 __device__ __forceinline__ void gstore(T FWDMI_GLOBAL* p, const Pack<T, N>& r) {
   if constexpr (N == 1) {

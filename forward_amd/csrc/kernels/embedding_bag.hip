@@ -58,6 +58,8 @@ constexpr int kUnroll = FWDMI_BAG_UNROLL;  // row loads in flight per lane
 // All loads of a lane's share (up to four vectors, the two ends) are issued before the first of
 // them is used: the workgroup waits for memory once, not once per vector and once per end (a run of
 // 1830 ids is two vectors for most lanes, and most runs start and end off a 16-byte boundary).
+// The vectors are loaded with the non-temporal hint: ids and weights are read once, and 111 MB of
+// them per launch of the 26-table configuration otherwise displace table rows in L2 (0.4229 -> 0.4220 ms).
 template <typename T, typename Put>
 __device__ __forceinline__ void stream_in(const T FWDMI_GLOBAL* first, int n, int tid, int lanes, Put put) {
   constexpr int kPer = 16 / (int)sizeof(T);
@@ -84,7 +86,7 @@ __device__ __forceinline__ void stream_in(const T FWDMI_GLOBAL* first, int n, in
 #pragma unroll
     for (int k = 0; k < kAhead; ++k) {
       const int v = v0 + k * lanes;
-      if (v < n_vec) p[k] = gload<T, kPer>(first + head + v * kPer);
+      if (v < n_vec) p[k] = gload_stream<T, kPer>(first + head + v * kPer);
     }
 #pragma unroll
     for (int k = 0; k < kAhead; ++k) {

@@ -301,6 +301,7 @@ def cpu_baseline(wl, tabs_dev, n_cpu_bags, torch):
         torch.set_num_threads(n)
         lt["threads_%d" % n] = total_bags / timed(run_torch, budget_s=6.0)
     torch.set_num_threads(cores)
+    lt_out = run_torch().numpy()
     res = {"value": lt["threads_%d" % cores], "unit": "bags/s", "cores": cores, "kind": "libtorch_cpu",
            "what": "26 x torch.nn.functional.embedding_bag(mode='sum') + torch.cat on CPU tensors (fp16 tables, "
                    "int32 ids): the ground truth of the reference's unit tests",
@@ -316,8 +317,18 @@ def cpu_baseline(wl, tabs_dev, n_cpu_bags, torch):
         pass
     log("cpu baseline: os.cpu_count()=%d, sched affinity=%d, OMP_NUM_THREADS=%s, threads used=%d" %
         (threads["os_cpu_count"], threads["sched_affinity"], threads["omp_num_threads_env"], cores))
-    # the oracle's output doubles as a check of the whole GPU result
-    return res, out, nb
+    # the oracle's output doubles as a check of the whole GPU result; libtorch's own result goes with it
+    return res, out, nb, lt_out
+
+
+def compare_with_libtorch(got, want, what="the whole fp16 result against libtorch's fp16 result, element by element"):
+    """A GPU launch's fp16 result against libtorch CPU's on the same inputs (the ground truth the reference's
+    unit tests use), at the stated bar for fp16 after fp32 accumulation: abs 1e-2 / rel 5e-3."""
+    g, w = got.astype(np.float32), want.astype(np.float32)
+    diff = np.abs(g - w)
+    return {"elements": int(g.size), "max_abs_diff": float(diff.max()), "differing_elements": int((diff > 0).sum()),
+            "within_abs_1e-2_rel_5e-3": bool((diff <= 1e-2 + 5e-3 * np.abs(w)).all()),
+            "what": what}
 
 
 def copy_bandwidth(torch):
@@ -356,6 +367,22 @@ def cpu_bert(torch, wl, threads):
         res["threads_%d" % n] = wl.n_tokens / float(np.median(ts))
     torch.set_num_threads(threads[0])
     return res
+
+
+def bert_libtorch_fp32(torch, wl):
+    """The same stage through libtorch CPU in fp32 on the workload's fp16 parameters (embedding x3 + add +
+    layer_norm, then the residual / bias add + layer_norm where the workload has one): what the GPU result
+    is compared with.  Returns (first stage, final stage or None)."""
+    F = torch.nn.functional
+    tw, tp, tt = (torch.from_numpy(a).float() for a in (wl.word, wl.pos, wl.tok))
+    ids, seg = torch.from_numpy(wl.input_ids).long(), torch.from_numpy(wl.segment_ids).long()
+    S, H = wl.input_ids.shape[0], wl.word.shape[1]
+    g, b = torch.from_numpy(wl.gamma).float(), torch.from_numpy(wl.beta).float()
+    e = F.layer_norm(F.embedding(ids, tw) + tp[:S].unsqueeze(1) + F.embedding(seg, tt), (H,), g, b, wl.eps)
+    if wl.skip is None:
+        return e.numpy(), None
+    sk, bi, g2, b2 = (torch.from_numpy(a).float() for a in (wl.skip, wl.skip_bias, wl.skip_gamma, wl.skip_beta))
+    return e.numpy(), F.layer_norm(e + sk + bi, (H,), g2, b2, wl.eps).numpy()
 
 
 def plugin_level(torch, wl, tabs, idx, off, want):
@@ -529,6 +556,9 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
         if with_cpu:
             cores = host_threads()["threads_used"]
             ex[name.split("_")[0] + "_libtorch_cpu_tokens_per_s"] = cpu_bert(torch, wl, tuple(sorted({cores, 1}, reverse=True)))
+            ref1, ref2 = bert_libtorch_fp32(torch, wl)
+            ex[name]["gpu_vs_libtorch_cpu_fp32"] = compare_with_libtorch(
+                out.cpu().numpy(), ref1, "the whole fp16 result against libtorch's fp32 evaluation of the same fp16 parameters")
         if wl.skip is not None:
             x, sk = out, dev(wl.skip)
             g, b, bi = f32(wl.skip_gamma), f32(wl.skip_beta), f32(wl.skip_bias)
@@ -537,6 +567,9 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
             ms = time_graph(torch, fn2)
             ex["config5_skip_layer_norm"] = {"tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
                                              "algorithmic_GBs": wl.skip_algorithmic_bytes() / (ms * 1e-3) / 1e9}
+            if with_cpu:   # the chain EmbLayerNorm -> SkipLayerNorm against libtorch's
+                ex["config5_skip_layer_norm"]["gpu_vs_libtorch_cpu_fp32"] = compare_with_libtorch(
+                    o2.cpu().numpy(), ref2, "the whole fp16 result of the two-stage chain against libtorch's fp32 evaluation")
             # yardsticks: torch's add on the same tensors (the same traffic, no reduction) and
             # PyTorch-ROCm's own GPU kernels for the same stage (add + bias, then layer_norm)
             ms_add = time_graph(torch, lambda: torch.add(x, sk, out=o2))
@@ -1075,12 +1108,13 @@ def main():
         del src, dst
     if not args.no_cpu:
         t1 = time.time()
-        cpu, cpu_out, nb = cpu_baseline(wls[checked_batch], tabs, args.cpu_bags, torch)
+        cpu, cpu_out, nb, lt_out = cpu_baseline(wls[checked_batch], tabs, args.cpu_bags, torch)
         cpu["gpu_matches_oracle_on_sample"] = bool(np.array_equal(gpu_out_checked[:nb].view(np.uint16),
                                                                   cpu_out.view(np.uint16)))
         cpu["checked"] = "the output of the last timed step (batch %d of %d) against the oracle, bit for bit" % (
             checked_batch, n_batches)
-        del gpu_out_checked, cpu_out
+        cpu["gpu_vs_libtorch_cpu"] = compare_with_libtorch(gpu_out_checked[:nb], lt_out)
+        del gpu_out_checked, cpu_out, lt_out
         result["cpu_baseline"] = cpu
         log("cpu baseline leg %.1fs" % (time.time() - t1))
     if not args.no_extra:

@@ -321,13 +321,16 @@ def cpu_baseline(wl, tabs_dev, n_cpu_bags, torch):
     return res, out, nb, lt_out
 
 
-def compare_with_libtorch(got, want, what="the whole fp16 result against libtorch's fp16 result, element by element"):
+def compare_with_libtorch(got, want, what="the whole fp16 result against libtorch's fp16 result, element by element",
+                          fp32=False):
     """A GPU launch's fp16 result against libtorch CPU's on the same inputs (the ground truth the reference's
-    unit tests use), at the stated bar for fp16 after fp32 accumulation: abs 1e-2 / rel 5e-3."""
+    unit tests use), at the stated bar: fp16 after fp32 accumulation abs 1e-2 / rel 5e-3, fp32 rel 1e-5 (with the
+    same figure as absolute floor for sums that cancel)."""
     g, w = got.astype(np.float32), want.astype(np.float32)
     diff = np.abs(g - w)
     return {"elements": int(g.size), "max_abs_diff": float(diff.max()), "differing_elements": int((diff > 0).sum()),
-            "within_abs_1e-2_rel_5e-3": bool((diff <= 1e-2 + 5e-3 * np.abs(w)).all()),
+            ("within_rel_1e-5" if fp32 else "within_abs_1e-2_rel_5e-3"):
+                bool((diff <= (1e-5 + 1e-5 * np.abs(w) if fp32 else 1e-2 + 5e-3 * np.abs(w))).all()),
             "what": what}
 
 
@@ -597,6 +600,11 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
     out = torch.empty((wl.n_bags, wl.table.shape[1]), dtype=tb.dtype, device="cuda")
     ms = time_graph(torch, lambda: ops.embedding_bag(tb, ix, of, "sum", out=out))
     ex["config1_sum_fp32_int64"] = {"bags_per_s": wl.n_bags / (ms * 1e-3), "ms": ms}
+    cpu_bag = lambda w: torch.nn.functional.embedding_bag(torch.from_numpy(w.indices).long(), torch.from_numpy(w.table),
+                                                          torch.from_numpy(w.offsets).long(), mode="sum").numpy()
+    if with_cpu:
+        ex["config1_sum_fp32_int64"]["gpu_vs_libtorch_cpu"] = compare_with_libtorch(
+            out.cpu().numpy(), cpu_bag(wl), "the whole fp32 result against libtorch's, element by element", fp32=True)
     for tdt, tname in ((np.float32, "fp32"), (np.float16, "fp16")):
         wl = workloads.config2(table_dtype=tdt)
         tb, ix, of = dev(wl.table), dev(wl.indices), dev(wl.offsets)
@@ -605,6 +613,10 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
         ms = time_graph(torch, fn)
         ex["config2_sum_%s_int32" % tname] = {"bags_per_s": wl.n_bags / (ms * 1e-3), "ms": ms,
                                               "algorithmic_GBs": wl.algorithmic_bytes() / (ms * 1e-3) / 1e9}
+        if with_cpu:
+            ex["config2_sum_%s_int32" % tname]["gpu_vs_libtorch_cpu"] = compare_with_libtorch(
+                out.cpu().numpy(), cpu_bag(wl), "the whole %s result against libtorch's, element by element" % tname,
+                fp32=tdt == np.float32)
         ix64, of64 = ix.long(), of.long()
         try:
             ms_t = time_graph(torch, lambda: torch.nn.functional.embedding_bag(ix64, tb, of64, mode="sum"))

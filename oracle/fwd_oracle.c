@@ -35,6 +35,10 @@
  *   embedding bag sum        pinned: reference-held tables + inputs (embedding_bag.pth,
  *                            dlrm.pth), numpy gather+sum, libtorch CPU
  *   mean / max / weights     pinned: libtorch CPU on seeded inputs, hand-worked NaN/tie cases
+ *                            (equal bit for bit, fp32 and fp16 tables, except the mean over an
+ *                            fp16 table: libtorch's CPU kernel rounds the sum to fp16 and divides
+ *                            that, this file divides the fp32 sum and rounds once; at most one
+ *                            fp16 unit apart, inside the fp16 bar)
  *   fixed-length / gather    pinned: numpy fancy indexing
  *   layer norm family        pinned: float64 closed form (numpy), libtorch CPU layer_norm,
  *                            standardisation invariants

@@ -55,6 +55,34 @@ def test_config2_scaled(oracle, tdt, idt, mode):
         assert_bits_equal(host(run_bag(wl.table, wl.indices, wl.offsets, m)), want, "max, values only")
 
 
+@pytest.mark.parametrize("tdt", [np.float32, np.float16])
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+@pytest.mark.parametrize("mode", ["sum", "mean", "max", "wsum"])
+def test_config2_scaled_against_libtorch_cpu_itself(tdt, idt, mode):
+    """The same launches against torch.nn.functional.embedding_bag on CPU tensors, run here and now (the
+    ground truth the reference's unit tests use), without the oracle in between: values within the
+    stated bar and in fact equal bit for bit, except the mean over an fp16 table (see below)."""
+    weighted = mode == "wsum"
+    m = "sum" if weighted else mode
+    wl = workloads.config2(variant=2, table_dtype=tdt, index_dtype=idt, mode=m, weighted=weighted, rows=60000)
+    psw = None if wl.per_sample_weights is None else torch.from_numpy(wl.per_sample_weights)
+    try:
+        ref = torch.nn.functional.embedding_bag(torch.from_numpy(wl.indices), torch.from_numpy(wl.table),
+                                                torch.from_numpy(wl.offsets), mode=m, per_sample_weights=psw)
+    except RuntimeError as e:   # a type / mode pair this libtorch build has no CPU kernel for
+        pytest.skip("libtorch CPU: %s" % str(e).splitlines()[0])
+    got = host(run_bag(wl.table, wl.indices, wl.offsets, m, wl.per_sample_weights))
+    assert_close(got, ref.numpy(), tdt, scale=0.05)
+    if mode == "mean" and tdt == np.float16:
+        # libtorch's CPU kernel rounds the bag's sum to fp16 and divides that; the launch divides the fp32
+        # sum and rounds once.  One fp16 unit apart at most, in about a quarter of the elements.
+        a, b = got.view(np.int16).astype(np.int32), ref.numpy().view(np.int16).astype(np.int32)
+        key = lambda v: np.where(v < 0, -(v & 0x7fff), v)     # fp16 bit patterns in value order
+        assert np.abs(key(a) - key(b)).max() <= 1
+    else:
+        assert_bits_equal(got, ref.numpy(), "%s against libtorch CPU" % mode)
+
+
 def test_max_ties_nan_and_empty_bags_match_libtorch_vectors(torch_vectors):
     """The committed libtorch CPU vectors (first maximum wins, NaN never replaces a value, a NaN
     first element stays, argmax is the row id, empty bags give 0 / 0) through the HIP path."""

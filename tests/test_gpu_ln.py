@@ -55,6 +55,17 @@ def test_config5_emb_then_skip_layer_norm(oracle, dtype):
     # second stage checked on the GPU's own first-stage output, so errors do not compound
     want = oracle.skip_layer_norm(host(emb), wl.skip_gamma, wl.skip_beta, skip=wl.skip, bias=wl.skip_bias, eps=wl.eps)
     assert_close(host(out), want, dtype)
+    # next to the oracle: libtorch CPU itself on the same parameters (embedding x3 + add + layer_norm, then
+    # the residual / bias add + layer_norm), evaluated in fp32
+    Fn = torch.nn.functional
+    S, H = wl.input_ids.shape[0], wl.word.shape[1]
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).float()
+    e = Fn.layer_norm(Fn.embedding(torch.from_numpy(wl.input_ids).long(), t(wl.word)) + t(wl.pos)[:S].unsqueeze(1)
+                      + Fn.embedding(torch.from_numpy(wl.segment_ids).long(), t(wl.tok)), (H,), t(wl.gamma), t(wl.beta),
+                      wl.eps)
+    assert_close(host(emb), e.numpy(), dtype)
+    ref = Fn.layer_norm(e + t(wl.skip) + t(wl.skip_bias), (H,), t(wl.skip_gamma), t(wl.skip_beta), wl.eps)
+    assert_close(host(out), ref.numpy(), dtype, scale=4.0)
 
 
 @pytest.mark.parametrize("ld,dtype", [(1, np.float32), (7, np.float32), (10, np.float32), (32, np.float16),

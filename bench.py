@@ -369,7 +369,7 @@ def cpu_bert(torch, wl, threads):
             ts.append(time.perf_counter() - t0)
         res["threads_%d" % n] = wl.n_tokens / float(np.median(ts))
     torch.set_num_threads(threads[0])
-    return res
+    return res, run().numpy()
 
 
 def bert_libtorch_fp32(torch, wl):
@@ -558,8 +558,12 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
                     "algorithmic_GBs": wl.emb_algorithmic_bytes() / (ms * 1e-3) / 1e9}
         if with_cpu:
             cores = host_threads()["threads_used"]
-            ex[name.split("_")[0] + "_libtorch_cpu_tokens_per_s"] = cpu_bert(torch, wl, tuple(sorted({cores, 1}, reverse=True)))
+            ex[name.split("_")[0] + "_libtorch_cpu_tokens_per_s"], native = cpu_bert(
+                torch, wl, tuple(sorted({cores, 1}, reverse=True)))
             ref1, ref2 = bert_libtorch_fp32(torch, wl)
+            if wl.skip is None:   # (with a second stage, libtorch's fp16 result is that stage's: compared there)
+                ex[name]["gpu_vs_libtorch_cpu_native_fp16"] = compare_with_libtorch(
+                    out.cpu().numpy(), native, "against libtorch's fp16 path, which rounds after every operation")
             ex[name]["gpu_vs_libtorch_cpu_fp32"] = compare_with_libtorch(
                 out.cpu().numpy(), ref1, "the whole fp16 result against libtorch's fp32 evaluation of the same fp16 parameters")
         if wl.skip is not None:
@@ -570,7 +574,9 @@ def extra_measurements(torch, ops, workloads, steps, with_cpu=True):
             ms = time_graph(torch, fn2)
             ex["config5_skip_layer_norm"] = {"tokens_per_s": wl.n_tokens / (ms * 1e-3), "ms": ms,
                                              "algorithmic_GBs": wl.skip_algorithmic_bytes() / (ms * 1e-3) / 1e9}
-            if with_cpu:   # the chain EmbLayerNorm -> SkipLayerNorm against libtorch's
+            if with_cpu:   # the chain EmbLayerNorm -> SkipLayerNorm against libtorch's, fp32 and its own fp16 path
+                ex["config5_skip_layer_norm"]["gpu_vs_libtorch_cpu_native_fp16"] = compare_with_libtorch(
+                    o2.cpu().numpy(), native, "against libtorch's fp16 path, which rounds after every operation")
                 ex["config5_skip_layer_norm"]["gpu_vs_libtorch_cpu_fp32"] = compare_with_libtorch(
                     o2.cpu().numpy(), ref2, "the whole fp16 result of the two-stage chain against libtorch's fp32 evaluation")
             # yardsticks: torch's add on the same tensors (the same traffic, no reduction) and

@@ -57,6 +57,9 @@ def parse():
                          "replays the same batch")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU: write profiles/traffic.json from two rocprofv3 --pmc counter_collection CSVs")
+    ap.add_argument("--record-l2", metavar="HIT_MISS_CSV",
+                    help="with --record-traffic: also the L2 hit rate of the launch, from a rocprofv3 --pmc TCC_HIT_sum "
+                         "TCC_MISS_sum counter_collection CSV of the same batch mode")
     ap.add_argument("--workload", default="config4", choices=["config4"])
     ap.add_argument("--tables", type=int, default=26, help="debug only: fewer tables (not the named config)")
     ap.add_argument("--bags", type=int, default=65536, help="debug only: smaller batch (not the named config)")
@@ -141,7 +144,7 @@ def load_traffic(section):
     return dict(t[section], kernel_source_sha256=t["kernel_source_sha256"])
 
 
-def record_traffic(fetch_csv, write_csv, batches):
+def record_traffic(fetch_csv, write_csv, batches, l2_csv=None):
     """profiles/traffic.json from two rocprofv3 counter CSVs (FETCH_SIZE / WRITE_SIZE, KiB per
     dispatch).  Each counter is scaled by what it reads for the 1 GiB device copy of the same run
     (--copy-calibration: 1 048 576 KiB read and as many written).  The counters sit at the L2's
@@ -181,6 +184,11 @@ def record_traffic(fetch_csv, write_csv, batches):
         "fetch_bytes": int(round(fetch * fs * 1024)), "write_bytes": int(round(write * ws * 1024)),
     }
     sec["bytes_per_launch"] = sec["fetch_bytes"] + sec["write_bytes"]
+    if l2_csv:
+        hit, _, nh = per_kernel(l2_csv, "TCC_HIT_sum")
+        miss, _, _ = per_kernel(l2_csv, "TCC_MISS_sum")
+        sec["l2_hits"], sec["l2_misses"], sec["l2_hit_rate"] = hit, miss, hit / (hit + miss)
+        sec["dispatches"].append(nh)
     out = {}
     if os.path.exists(TRAFFIC_JSON):
         with open(TRAFFIC_JSON) as f:
@@ -954,7 +962,7 @@ def lru_sim(workloads, capacities=(8192, 12288, 16384, 32768)):
 def main():
     args = parse()
     if args.record_traffic:
-        record_traffic(*args.record_traffic, batches=args.batches)
+        record_traffic(*args.record_traffic, batches=args.batches, l2_csv=args.record_l2)
         return
     if args.lru_sim:
         sys.path.insert(0, ROOT)
@@ -1094,6 +1102,9 @@ def main():
         r["frac_hbm_side_is"] = "traffic / kernel time / HBM peak: what crosses the L2 boundary against the 8 TB/s ceiling"
         r["refetch_ratio"] = traffic["fetch_bytes"] / float(
             comp_bytes - len(wl.rows) * wl.n_bags * wl.dim * 2)   # fetched / (distinct rows + ids + offsets), batch 0
+        if "l2_hit_rate" in traffic:
+            r["l2_hit_rate"] = traffic["l2_hit_rate"]
+            r["l2_hit_rate_is"] = "TCC_HIT_sum / (TCC_HIT_sum + TCC_MISS_sum) of this launch (rocprofv3, a pass of its own)"
         r["traffic_kernel_source_sha256"] = traffic["kernel_source_sha256"]
     else:
         result["roofline"]["frac_hbm_side"] = None

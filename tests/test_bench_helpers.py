@@ -42,6 +42,15 @@ def test_record_traffic_scales_by_the_calibration_copy_and_keeps_one_section_per
     assert sec["fetch_bytes"] == int(round(500001.0 * 2 * 1024)) and sec["write_bytes"] == 400000 * 1024
     assert sec["bytes_per_launch"] == sec["fetch_bytes"] + sec["write_bytes"]
     assert t["kernel_source_sha256"] == bench.kernel_source_hash() and "same_batch" not in t
+    # the launch's L2 hit rate from a third counter pass goes into the same section
+    h = str(tmp_path / "h.csv")
+    with open(h, "w") as fh:
+        fh.write("Kernel_Name,Counter_Name,Counter_Value\n")
+        for name, vals in (("TCC_HIT_sum", [300.0, 500.0]), ("TCC_MISS_sum", [100.0, 100.0])):
+            for v in vals:
+                fh.write("fwdmi::bag_reduce_kernel<x>,%s,%s\n" % (name, v))
+    bench.record_traffic(f, w, batches=8, l2_csv=h)
+    assert json.load(open(bench.TRAFFIC_JSON))["rotating_batches"]["l2_hit_rate"] == 400.0 / 500.0
     bench.record_traffic(f, w, batches=1)                                                # the other mode joins it
     t = json.load(open(bench.TRAFFIC_JSON))
     assert set(t) >= {"rotating_batches", "same_batch"} and t["same_batch"]["batches"] == 1
